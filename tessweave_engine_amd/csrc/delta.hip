@@ -1,0 +1,208 @@
+// The gated delta rule: a recurrent mixer whose state is corrected towards each new value before it is read.
+//
+//   per value head h (its query/key head is h / (H / G)), S: [D][E] float32, carried from step to step:
+//     q~ = q / sqrt(sum q^2 + 1e-6) * q_scale        k~ = k / sqrt(sum k^2 + 1e-6)
+//     beta = sigmoid(b)      g = exp(-exp(A_log_h) * softplus(a + dt_bias_h))
+//     S <- g S;   u = beta (v - S^T k~);   S <- S + k~ u^T;   o = S^T q~          (the read-out sees the token's write)
+//
+// q, k, v arrive in float32 (a short convolution's result), b and a are columns of a float32 projection; the unit
+// norms, the gates, the state and every product with it are float32. A step's rows of one sequence are walked in
+// order from the request's state, which the same lanes read at the start and write at the end: nothing depends on
+// how a prompt was cut.
+//
+// A workgroup owns 64 value columns of one (sequence, head). A wave holds 16 of them: lane = 4 * column + slice,
+// and a lane keeps the quarter `slice` of its column of S in registers (DPL elements), so both products of a token
+// are DPL multiply-adds and two lane swaps inside a quad. The state lies in memory as [H][E][Dk] (a column of S is
+// contiguous), Dk = 4 * DPL. Tokens are staged in LDS in chunks: the waves share a chunk's tokens out, norm q and k,
+// form beta and g, then all walk the chunk.
+#include "tw_common.h"
+
+#define TW_DELTA_CHUNK 16
+
+struct DeltaArgs {
+  const float* qkv; long ld_qkv;      // q of key head j at q_col + j * D, k at k_col + j * D, v of head h at v_col + h * E
+  int q_col, k_col, v_col;
+  const float* ab; long ld_ab;        // b of head h at b_col + h, a at a_col + h
+  int b_col, a_col;
+  const float* A_log; const float* dt_bias;   // [H]
+  float* state;                       // [requests][H][E][Dk]
+  const int* q_start; const int* state_slots;
+  float* out; long ld_out;            // float32 [n][>= H * E]: head h at h * E
+  int H, G, D, E, Dk;
+  float q_scale;
+};
+
+template <int CTRL>
+__device__ __forceinline__ float delta_quad_swap(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// sum over the four lanes of a quad; every lane gets it
+__device__ __forceinline__ float delta_quad_sum(float v) {
+  v += delta_quad_swap<0xB1>(v);      // lanes 1 0 3 2
+  v += delta_quad_swap<0x4E>(v);      // lanes 2 3 0 1
+  return v;
+}
+
+__device__ __forceinline__ float delta_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+template <int DPL>
+__global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) {
+  constexpr int SL = DPL + 4;                        // a slice's stride in LDS: the four slices of a quad meet different banks
+  constexpr int ROW = 4 * SL;
+  __shared__ __attribute__((aligned(16))) float q_s[TW_DELTA_CHUNK][ROW];
+  __shared__ __attribute__((aligned(16))) float k_s[TW_DELTA_CHUNK][ROW];
+  __shared__ float v_s[TW_DELTA_CHUNK][64];
+  __shared__ float gate_s[TW_DELTA_CHUNK][2];        // beta, g
+  const int blocks_e = (a.E + 63) / 64;
+  const int eb = blockIdx.x % blocks_e, head = blockIdx.x / blocks_e;
+  const int s = seq0 + blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int slice = lane & 3;
+  const int e = eb * 64 + wave * 16 + (lane >> 2);
+  const bool live = e < a.E;
+  const int kh = head / (a.H / a.G);
+  const int first = a.q_start[s], last = a.q_start[s + 1];
+  float* S_mem = a.state + (((size_t)a.state_slots[s] * a.H + head) * a.E + (live ? e : 0)) * a.Dk + slice * DPL;
+  const bool held = live && slice * DPL < a.Dk;      // (Dk may be shorter than 4 * DPL: the last slices then hold nothing)
+  float S[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; i += 4) {
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (held && slice * DPL + i < a.Dk) v = *reinterpret_cast<const f32x4*>(S_mem + i);
+    S[i] = v[0]; S[i + 1] = v[1]; S[i + 2] = v[2]; S[i + 3] = v[3];
+  }
+  const float rate = -expf(a.A_log[head]);
+  const float dt_bias = a.dt_bias[head];
+  for (int t0 = first; t0 < last; t0 += TW_DELTA_CHUNK) {
+    const int nt = min(TW_DELTA_CHUNK, last - t0);
+    __syncthreads();                                 // the chunk before has been walked by every wave
+    for (int i = wave; i < nt; i += 4) {
+      const float* row = a.qkv + (size_t)(t0 + i) * a.ld_qkv;
+      const float* qr = row + a.q_col + (size_t)kh * a.D;
+      const float* kr = row + a.k_col + (size_t)kh * a.D;
+      float qv[4], kv[4], qq = 0.f, kk = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = lane + 64 * j;
+        qv[j] = d < a.D ? qr[d] : 0.f;
+        kv[j] = d < a.D ? kr[d] : 0.f;
+        qq = __fmaf_rn(qv[j], qv[j], qq);
+        kk = __fmaf_rn(kv[j], kv[j], kk);
+      }
+      qq = tw_wave_sum(qq);
+      kk = tw_wave_sum(kk);
+      const float qn = a.q_scale / sqrtf(qq + 1e-6f), kn = 1.f / sqrtf(kk + 1e-6f);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = lane + 64 * j;
+        if (d < 4 * DPL) {
+          q_s[i][(d / DPL) * SL + d % DPL] = qv[j] * qn;
+          k_s[i][(d / DPL) * SL + d % DPL] = kv[j] * kn;
+        }
+      }
+      const int ev = eb * 64 + lane;
+      v_s[i][lane] = ev < a.E ? row[a.v_col + (size_t)head * a.E + ev] : 0.f;
+      if (lane == 0) {
+        const float* ab = a.ab + (size_t)(t0 + i) * a.ld_ab;
+        const float b = ab[a.b_col + head], x = ab[a.a_col + head];
+        gate_s[i][0] = 1.f / (1.f + expf(-b));
+        gate_s[i][1] = expf(rate * delta_softplus(x + dt_bias));
+      }
+    }
+    __syncthreads();
+    for (int i = 0; i < nt; ++i) {
+      const float* kp = &k_s[i][slice * SL];
+      const float* qp = &q_s[i][slice * SL];
+      const float beta = gate_s[i][0], g = gate_s[i][1];
+      float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+      for (int j = 0; j < DPL; j += 4) {
+        const f32x4 kq = *reinterpret_cast<const f32x4*>(kp + j);
+        d0 = __fmaf_rn(S[j], kq[0], d0);
+        d1 = __fmaf_rn(S[j + 1], kq[1], d1);
+        d2 = __fmaf_rn(S[j + 2], kq[2], d2);
+        d3 = __fmaf_rn(S[j + 3], kq[3], d3);
+      }
+      const float dot = delta_quad_sum((d0 + d1) + (d2 + d3));
+      const float u = beta * (v_s[i][wave * 16 + (lane >> 2)] - g * dot);
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+      for (int j = 0; j < DPL; j += 4) {
+        const f32x4 kq = *reinterpret_cast<const f32x4*>(kp + j);
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(qp + j);
+        S[j] = __fmaf_rn(kq[0], u, g * S[j]);
+        S[j + 1] = __fmaf_rn(kq[1], u, g * S[j + 1]);
+        S[j + 2] = __fmaf_rn(kq[2], u, g * S[j + 2]);
+        S[j + 3] = __fmaf_rn(kq[3], u, g * S[j + 3]);
+        o0 = __fmaf_rn(S[j], qq[0], o0);
+        o1 = __fmaf_rn(S[j + 1], qq[1], o1);
+        o2 = __fmaf_rn(S[j + 2], qq[2], o2);
+        o3 = __fmaf_rn(S[j + 3], qq[3], o3);
+      }
+      const float o = delta_quad_sum((o0 + o1) + (o2 + o3));
+      if (live && slice == 0) a.out[(size_t)(t0 + i) * a.ld_out + (size_t)head * a.E + e] = o;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < DPL; i += 4)
+    if (held && slice * DPL + i < a.Dk) *reinterpret_cast<f32x4*>(S_mem + i) = f32x4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+}
+
+extern "C" int tw_delta_rule(const float* qkv, long ld_qkv, int q_col, int k_col, int v_col, const float* ab, long ld_ab,
+                             int b_col, int a_col, const float* A_log, const float* dt_bias, float* state,
+                             const int* q_start, const int* state_slots, float* out, long ld_out, int seq0, int n_seqs,
+                             int H, int G, int D, int E, int Dk, float q_scale, hipStream_t stream) {
+  TW_REQUIRE(qkv && ab && A_log && dt_bias && state && q_start && state_slots && out);
+  TW_REQUIRE(H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && E > 0 && Dk >= D && Dk % 4 == 0 && Dk <= 256);
+  TW_REQUIRE(seq0 >= 0 && n_seqs >= 0 && ld_out >= (long)H * E && (uintptr_t)state % 16 == 0);
+  TW_REQUIRE(q_col >= 0 && k_col >= 0 && v_col >= 0 && b_col >= 0 && a_col >= 0);
+  TW_REQUIRE(ld_qkv >= (long)max(q_col, k_col) + (long)G * D && ld_qkv >= (long)v_col + (long)H * E);
+  TW_REQUIRE(ld_ab >= (long)max(a_col, b_col) + H);
+  if (n_seqs == 0) return 0;
+  DeltaArgs a{qkv, ld_qkv, q_col, k_col, v_col, ab, ld_ab, b_col, a_col, A_log, dt_bias, state, q_start, state_slots,
+              out, ld_out, H, G, D, E, Dk, q_scale};
+  const dim3 grid(H * tw_div_up(E, 64), n_seqs);
+  if (Dk <= 16) delta_walk_kernel<4><<<grid, 256, 0, stream>>>(a, seq0);
+  else if (Dk <= 32) delta_walk_kernel<8><<<grid, 256, 0, stream>>>(a, seq0);
+  else if (Dk <= 64) delta_walk_kernel<16><<<grid, 256, 0, stream>>>(a, seq0);
+  else if (Dk <= 128) delta_walk_kernel<32><<<grid, 256, 0, stream>>>(a, seq0);
+  else delta_walk_kernel<64><<<grid, 256, 0, stream>>>(a, seq0);
+  return TW_LAUNCH_RESULT();
+}
+
+// out[n][h * E + e] = o[n][h * E + e] / sqrt(mean_e(o^2) + eps) * weight[e] * silu(gate[n][h * E + e]), rounded to the
+// compute type: a unit norm per head with one weight vector shared by the heads, times a gate. One wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, long ld_o, const float* __restrict__ gate,
+                                                             long ld_g, const float* __restrict__ weight, T* __restrict__ out,
+                                                             long ld_out, int n, int H, int E, float eps) {
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (unit >= n * H) return;
+  const int lane = threadIdx.x & 63;
+  const int row = unit / H, head = unit % H;
+  const float* src = o + (size_t)row * ld_o + (size_t)head * E;
+  float ss = 0.f;
+  for (int e = lane; e < E; e += 64) ss = __fmaf_rn(src[e], src[e], ss);
+  ss = tw_wave_sum(ss);
+  const float rinv = 1.f / sqrtf(ss / (float)E + eps);
+  const float* g = gate + (size_t)row * ld_g + (size_t)head * E;
+  T* dst = out + (size_t)row * ld_out + (size_t)head * E;
+  for (int e = lane; e < E; e += 64) {
+    const float z = g[e];
+    dst[e] = tw_from_float<T>(src[e] * rinv * weight[e] * (z / (1.f + expf(-z))));
+  }
+}
+
+extern "C" int tw_head_norm_gate(int dtype, const float* o, long ld_o, const float* gate, long ld_g, const float* weight,
+                                 void* out, long ld_out, int n, int H, int E, float eps, hipStream_t stream) {
+  TW_REQUIRE(o && gate && weight && out && n >= 0 && H > 0 && E > 0 && eps > 0.f);
+  TW_REQUIRE(ld_o >= (long)H * E && ld_g >= (long)H * E && ld_out >= (long)H * E);
+  if (n == 0) return 0;
+  const int blocks = tw_div_up((long)n * H, 4);
+  if (dtype == TW_DTYPE_BF16)
+    head_norm_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(o, ld_o, gate, ld_g, weight, (bf16_t*)out, ld_out, n, H, E, eps);
+  else if (dtype == TW_DTYPE_F32)
+    head_norm_gate_kernel<float><<<blocks, 256, 0, stream>>>(o, ld_o, gate, ld_g, weight, (float*)out, ld_out, n, H, E, eps);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}

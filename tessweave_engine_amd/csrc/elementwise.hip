@@ -634,3 +634,73 @@ extern "C" int tw_silu_mul(int dtype, const void* gu, void* out, int n, int inte
     return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
 }
+
+// ---- the same with the limited swish: out[n, i] = glu(gu[n, i], gu[n, inter + i]) of TW_GLU_SWISH_LIMITED -----------
+template <typename T>
+__global__ void swish_limited_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int inter, float limit) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * inter) return;
+  const long row = i / inter;
+  const int col = (int)(i % inter);
+  float g = fminf(tw_to_float(gu[row * 2 * inter + col]), limit);
+  float u = fminf(fmaxf(tw_to_float(gu[row * 2 * inter + inter + col]), -limit), limit);
+  out[i] = tw_from_float<T>(g / (1.0f + expf(-1.702f * g)) * (u + 1.f));
+}
+
+extern "C" int tw_swish_limited_mul(int dtype, const void* gu, void* out, int n, int inter, float limit, hipStream_t stream) {
+  TW_REQUIRE(n >= 0 && inter > 0);
+  if (n == 0) return 0;
+  const int blocks = tw_div_up((long)n * inter, 256);
+  if (dtype == TW_DTYPE_F32)
+    swish_limited_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, n, inter, limit);
+  else if (dtype == TW_DTYPE_BF16)
+    swish_limited_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, inter, limit);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- two RMS norms of the same rows: out1 = unit(x) * w1, out2 = unit(x) * w2 (out2 and w2 may be null) --------------
+// For arrangements whose sublayers all read norms of the same stream: the row is read and its statistic formed once.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_pair_kernel(const float* __restrict__ x, const float* __restrict__ w1,
+                                                           const float* __restrict__ w2, T* __restrict__ out1,
+                                                           T* __restrict__ out2, int hidden, float eps) {
+  __shared__ float red[16];
+  const float* row = x + (size_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) ss = __fmaf_rn(row[c], row[c], ss);
+  ss = tw_block_sum(ss, red);
+  const float rinv = 1.f / sqrtf(ss / (float)hidden + eps);
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float u = row[c] * rinv;
+    out1[(size_t)blockIdx.x * hidden + c] = tw_from_float<T>(u * w1[c]);
+    if (out2) out2[(size_t)blockIdx.x * hidden + c] = tw_from_float<T>(u * w2[c]);
+  }
+}
+
+extern "C" int tw_rmsnorm_pair(int dtype, const float* x, const float* w1, const float* w2, void* out1, void* out2, int n,
+                               int hidden, float eps, hipStream_t stream) {
+  TW_REQUIRE(x && w1 && out1 && ((w2 != nullptr) == (out2 != nullptr)) && n >= 0 && hidden > 0 && eps > 0.f);
+  if (n == 0) return 0;
+  if (dtype == TW_DTYPE_F32)
+    rmsnorm_pair_kernel<float><<<n, 256, 0, stream>>>(x, w1, w2, (float*)out1, (float*)out2, hidden, eps);
+  else if (dtype == TW_DTYPE_BF16)
+    rmsnorm_pair_kernel<bf16_t><<<n, 256, 0, stream>>>(x, w1, w2, (bf16_t*)out1, (bf16_t*)out2, hidden, eps);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- x *= factor over a float32 buffer (a head whose logits carry a scale) ------------------------------------------
+__global__ void scale_values_kernel(float* __restrict__ x, long total, float factor) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) x[i] *= factor;
+}
+
+extern "C" int tw_scale_values(float* x, long total, float factor, hipStream_t stream) {
+  TW_REQUIRE(x && total >= 0);
+  if (total == 0) return 0;
+  scale_values_kernel<<<tw_div_up(total, 256), 256, 0, stream>>>(x, total, factor);
+  return TW_LAUNCH_RESULT();
+}

@@ -791,7 +791,7 @@ static int glu_layout(int shuffled, const T* A, long lda, const T* W, long ldw, 
 extern "C" int tw_linear_glu(int dtype, const void* A, long lda, const void* W, long ldw, int shuffled,
                              const float* bias, void* C, long ldc, int M, int N, int K, int force, int act,
                              float factor, hipStream_t stream) {
-  TW_REQUIRE(act == TW_GLU_SILU || act == TW_GLU_GELU_TANH);
+  TW_REQUIRE(act == TW_GLU_SILU || act == TW_GLU_GELU_TANH || act == TW_GLU_SWISH_LIMITED);
   const long code = tw_glu_code(act, factor);
   TW_REQUIRE(M >= 0 && N > 0 && N % 32 == 0 && K > 0 && lda >= K && ldc >= N / 2);
   TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K));

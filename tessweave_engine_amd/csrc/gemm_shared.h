@@ -10,8 +10,16 @@ __device__ __forceinline__ float tw_silu(float g) { return g / (1.0f + expf(-g))
 // activation the gate passes and a factor for the product: 0 is SiLU and 1 (what every caller before the second
 // activation passed); otherwise bits 32.. name the activation (1: the tanh form of gelu) and the low 32 bits are
 // the factor as a float. The factor is applied in float32 before the one rounding to the output type.
+// TW_GLU_SWISH_LIMITED reads the float as a limit L instead: with g' = min(g, L) and u' = clamp(u, -L, L) the result is
+// g' * sigmoid(1.702 g') * (u' + 1).
 #define TW_GLU_SILU 0
 #define TW_GLU_GELU_TANH 1
+#define TW_GLU_SWISH_LIMITED 2
+__device__ __forceinline__ float tw_swish_limited(float g, float u, float limit) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+}
 static inline long tw_glu_code(int act, float factor) {
   if (act == TW_GLU_SILU && factor == 1.0f) return 0;
   unsigned bits;
@@ -22,6 +30,7 @@ __device__ __forceinline__ float tw_glu(float g, float u, long code) {
   if (code == 0) return tw_silu(g) * u;
   const float factor = __uint_as_float((unsigned)(code & 0xffffffffL));
   const int act = (int)(code >> 32) - 1;
+  if (act == TW_GLU_SWISH_LIMITED) return tw_swish_limited(g, u, factor);
   const float a = act == TW_GLU_GELU_TANH ? 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)))
                                           : tw_silu(g);
   return factor * a * u;

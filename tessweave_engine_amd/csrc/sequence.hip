@@ -73,7 +73,17 @@ struct ConvArgs {
   float* out32; long ld_out32;        // float32, or null
   int n_seqs, C, K;
   float eps, identity;
+  int act;                            // 0: none; 1: SiLU of the result (after the bias), before the rounding
 };
+
+__device__ __forceinline__ float conv_act(float v, int act) { return act == 1 ? v / (1.f + expf(-v)) : v; }
+__device__ __forceinline__ f32x4 conv_act(f32x4 v, int act) {
+  if (act == 1) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = v[e] / (1.f + expf(-v[e]));
+  }
+  return v;
+}
 
 __device__ __forceinline__ f32x4 conv_load4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 __device__ __forceinline__ f32x4 conv_load4(const bf16_t* p) {
@@ -169,6 +179,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
           if (last && j >= 1) conv_store4(new_state + (size_t)(j - 1) * C + c, v[j]);
         }
       }
+      acc = conv_act(acc, a.act);
       if (a.out) conv_store4((OutT*)a.out + (size_t)row * a.ld_out + c, acc);
       if (a.out32) conv_store4(a.out32 + (size_t)row * a.ld_out32 + c, acc);
     }
@@ -193,6 +204,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
         if (last && j >= 1) new_state[(size_t)(j - 1) * C + c] = v[j];
       }
     }
+    acc = conv_act(acc, a.act);
     if (a.out) ((OutT*)a.out)[(size_t)row * a.ld_out + c] = tw_from_float<OutT>(acc);
     if (a.out32) a.out32[(size_t)row * a.ld_out32 + c] = acc;
   }
@@ -262,6 +274,7 @@ __global__ __launch_bounds__(256) void causal_conv_tile_kernel(ConvArgs a, int n
 #pragma unroll
       for (int j = 0; j < TW_CONV_MAX_TAPS; ++j)
         if (j == K - 1) acc += w[j] * cur;
+      acc = conv_act(acc, a.act);
       if (a.out) conv_store4((OutT*)a.out + (size_t)row * a.ld_out + c, acc);
       if (a.out32) conv_store4(a.out32 + (size_t)row * a.ld_out32 + c, acc);
       // shift: what met tap j + 1 meets tap j for the next row
@@ -305,8 +318,9 @@ extern "C" int tw_causal_conv(int dtype, int src_f32, const void* src, long ld_s
                               const float* taps, const float* bias, float identity, float* state,
                               const int* q_start, const int* kv_len, const int* state_slots, const int* phase,
                               void* out, long ld_out, float* out32, long ld_out32, int n_tokens, int n_seqs,
-                              int C, int K, float* row_scratch, hipStream_t stream) {
+                              int C, int K, float* row_scratch, int act, hipStream_t stream) {
   TW_REQUIRE(src && taps && state && q_start && kv_len && state_slots && phase && (out || out32));
+  TW_REQUIRE(act == 0 || act == 1);
   TW_REQUIRE(n_tokens >= 0 && n_seqs >= 1 && C > 0 && K >= 1 && K <= TW_CONV_MAX_TAPS);
   TW_REQUIRE(ld_src >= C && (!out || ld_out >= C) && (!out32 || ld_out32 >= C));
   TW_REQUIRE(!norm_w || src_f32);
@@ -319,7 +333,7 @@ extern "C" int tw_causal_conv(int dtype, int src_f32, const void* src, long ld_s
     row_rinv = row_scratch;
   }
   ConvArgs a{src, ld_src, norm_w, row_rinv, taps, bias, state, q_start, kv_len, state_slots, phase,
-             out, ld_out, out32, ld_out32, n_seqs, C, K, eps, identity};
+             out, ld_out, out32, ld_out32, n_seqs, C, K, eps, identity, act};
   const bool bf = dtype == TW_DTYPE_BF16;
   TW_REQUIRE(bf || dtype == TW_DTYPE_F32);
   // few rows (decode steps): the channels are shared out over several blocks a row

@@ -38,7 +38,7 @@ _SIGNATURES = {
     "tw_attn_prefill_workspace_floats": (L, [I, I, I, I]),
     "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P]),
     "tw_add_table_rows": (I, [I, P, P, P, I, I, I, P, P]),
-    "tw_causal_conv": (I, [I, I, P, L, P, F, P, P, F, P, P, P, P, P, P, L, P, L, I, I, I, I, P, P]),
+    "tw_causal_conv": (I, [I, I, P, L, P, F, P, P, F, P, P, P, P, P, P, L, P, L, I, I, I, I, P, I, P]),
     "tw_gated_recurrence_workspace_floats": (L, [I, I, I]),
     "tw_gated_recurrence": (I, [I, P, L, P, L, P, L, P, P, P, P, P, L, I, I, I, I, I, F, F, P, L, P]),
     "tw_block_diagonal": (I, [I, P, L, P, P, P, L, I, I, I, I, P]),
@@ -64,6 +64,14 @@ _SIGNATURES = {
     "tw_retention_workspace_floats": (L, [I, I, I, I, I]),
     "tw_retention": (I, [I, P, L, I, I, I, P, P, I, P, P, P, P, P, L, I, I, I, I, I, I, F, P, L, P]),
     "tw_unit_gate": (I, [I, P, L, P, L, P, L, I, I, I, I, F, P]),
+    "tw_swish_limited_mul": (I, [I, P, P, I, I, F, P]),
+    "tw_rmsnorm_pair": (I, [I, P, P, P, P, P, I, I, F, P]),
+    "tw_scale_values": (I, [P, L, F, P]),
+    "tw_delta_rule": (I, [P, L, I, I, I, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, I, I, F, P]),
+    "tw_head_norm_gate": (I, [I, P, L, P, L, P, P, L, I, I, I, F, P]),
+    "tw_moe_route": (I, [I, P, L, P, I, I, I, I, P, P, P]),
+    "tw_moe_capacity": (L, [L, I]),
+    "tw_moe_experts": (I, [I, P, L, P, P, I, I, I, P, P, P, I, I, I, F, P, P, P, P, P, P, I, P, L, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),
     "tw_sample_rows": (I, [P, L, I, I, P, P, P, P, P, L, P]),

@@ -282,13 +282,14 @@ def interleave_glu_rows(gate, up):
     return torch.stack([gate.reshape(n // 16, 16, *rest), up.reshape(n // 16, 16, *rest)], 1).reshape(2 * n, *rest).contiguous()
 
 
-GLU_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+GLU_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swish_limited": 2}
 
 
 def linear_glu(x, weight, out, bias=None, force=0, activation="silu", factor=1.0):
     """out[m, n/2] = factor * act(x @ gate.T) * (x @ up.T), weight [n, k] holding gate and up rows
     interleaved by `interleave_glu_rows` (row-major or shuffled); out has x's type. act is SiLU or the tanh
-    form of gelu; the factor is applied in float32 before the rounding."""
+    form of gelu; the factor is applied in float32 before the rounding. With "swish_limited" the factor is a limit L
+    instead: out = g' * sigmoid(1.702 g') * (u' + 1), g' = min(gate, L), u' = clamp(up, -L, L)."""
     _need(activation in GLU_ACTIVATIONS, f"activation must be one of {sorted(GLU_ACTIVATIONS)}")
     m, k, lda = _rows(x, "x")
     n, k2, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
@@ -511,16 +512,20 @@ def add_table_rows(x, table, ids, copy=None):
 CONV_MAX_TAPS = 8
 
 
+CONV_ACTIVATIONS = {None: 0, "silu": 1}
+
+
 def causal_conv(src, taps, state, q_start, kv_len, state_slots, phase, n_seqs, out=None, out32=None, norm_weight=None,
-                eps=0.0, bias=None, identity=0.0, row_scratch=None):
+                eps=0.0, bias=None, identity=0.0, row_scratch=None, activation=None):
     """Causal convolution over time on each channel, with the request's last inputs as state.
 
     v_t = src_t (or its RMS norm times norm_weight, for float32 rows); out_t = identity * v_t +
     sum_j taps[:, j] * v_(t - K + 1 + j) + bias. state float32 [requests, 2, max(K - 1, 1), C]: copy
     phase[s] is read, the other copy written. out has the compute type, out32 is float32; either may be None.
     row_scratch: float32 [>= n]; with a norm and many rows the rows' statistics are then formed once by a kernel of
-    their own.
+    their own. activation "silu": out_t passes SiLU before it is written (the state keeps the inputs v, as always).
     """
+    _need(activation in CONV_ACTIVATIONS, "a convolution's activation is None or 'silu'")
     n, C, ld_src = _rows(src, "src")
     K = taps.shape[1]
     _need(taps.dtype == torch.float32 and taps.is_contiguous() and taps.shape[0] == C, "taps must be float32 [C, K]")
@@ -555,7 +560,8 @@ def causal_conv(src, taps, state, q_start, kv_len, state_slots, phase, n_seqs, o
                                    _dev(state_slots, torch.int32, "state_slots"), _dev(phase, torch.int32, "phase"),
                                    _dev(out) if out is not None else None, ld_out,
                                    _dev(out32) if out32 is not None else None, ld_out32, n, int(n_seqs), C, K,
-                                   _dev(row_scratch, torch.float32, "row_scratch") if use_scratch else None, _stream()),
+                                   _dev(row_scratch, torch.float32, "row_scratch") if use_scratch else None,
+                                   CONV_ACTIVATIONS[activation], _stream()),
           "causal_conv")
 
 
@@ -1000,3 +1006,145 @@ def unit_gate(o, gate, out, heads, value_dim, value_dev, eps):
     check(library().tw_unit_gate(dtype_id(out.dtype), _dev(o), ld_o, _dev(gate), ld_g, _dev(out), ld_n, n, heads, int(value_dim),
                                  int(value_dev), float(eps), _stream()), "unit_gate")
     return out
+
+
+# ---- what the Rufusun design added ------------------------------------------------------------------------------
+
+def swish_limited_mul(gate_up, out, limit):
+    """out[n, i] = g' * sigmoid(1.702 g') * (u' + 1) with g' = min(gate_up[n, i], limit), u' = clamp(gate_up[n, inter + i],
+    -limit, limit): the limited swish where gate and up rows cannot be interleaved for the product's epilogue."""
+    n, inter = out.shape
+    _need(gate_up.is_contiguous() and out.is_contiguous() and tuple(gate_up.shape) == (n, 2 * inter) and gate_up.dtype == out.dtype,
+          "swish_limited_mul takes contiguous [n, 2 * inter] and [n, inter] of one type")
+    check(library().tw_swish_limited_mul(dtype_id(out.dtype), _dev(gate_up), _dev(out), n, inter, float(limit), _stream()),
+          "swish_limited_mul")
+    return out
+
+
+def rmsnorm_pair(x, weight1, eps, out1, weight2=None, out2=None):
+    """out1 = x * rsqrt(mean(x^2) + eps) * weight1 and, if asked for, out2 = the same rows times weight2: two norms of
+    the same float32 rows from one pass (the weights are float32 and hold every factor, a stored offset included)."""
+    _need(x.dim() == 2 and x.is_contiguous() and x.dtype == torch.float32, "rmsnorm_pair input must be contiguous float32 [n, hidden]")
+    n, hidden = x.shape
+    _need((weight2 is None) == (out2 is None), "a second weight and a second output come together")
+    for w, o in ((weight1, out1), (weight2, out2)):
+        if w is not None:
+            _need(w.numel() == hidden and w.is_contiguous() and o.is_contiguous() and tuple(o.shape) == (n, hidden)
+                  and o.dtype == out1.dtype, "rmsnorm_pair weights are [hidden], outputs contiguous [n, hidden] of one type")
+    check(library().tw_rmsnorm_pair(dtype_id(out1.dtype), _dev(x), _dev(weight1, torch.float32, "weight1"),
+                                    _dev(weight2, torch.float32, "weight2") if weight2 is not None else None, _dev(out1),
+                                    _dev(out2) if out2 is not None else None, n, hidden, float(eps), _stream()), "rmsnorm_pair")
+    return out1, out2
+
+
+def scale_values(x, factor):
+    """x *= factor in place (contiguous float32)."""
+    _need(x.is_contiguous() and x.dtype == torch.float32, "scale_values takes a contiguous float32 tensor")
+    check(library().tw_scale_values(_dev(x), x.numel(), float(factor), _stream()), "scale_values")
+    return x
+
+
+def delta_key_extent(dim):
+    """Elements a column of the delta rule's state holds on the device: the key size rounded up to a multiple of 4."""
+    return (int(dim) + 3) // 4 * 4
+
+
+def delta_rule(qkv, q_col, k_col, v_col, ab, b_col, a_col, A_log, dt_bias, state, q_start, state_slots, seq0, n_seqs, out,
+               kv_heads, dim, q_scale):
+    """The gated delta rule over sequences seq0 .. seq0 + n_seqs - 1, token by token from and to state float32
+    [requests, H, E, Dk] (a column of S is contiguous; Dk = delta_key_extent(dim)):
+
+        q~ = unit(q) * q_scale, k~ = unit(k) (unit: x / sqrt(sum x^2 + 1e-6)), beta = sigmoid(b),
+        g = exp(-exp(A_log) * softplus(a + dt_bias));  S <- g S;  u = beta (v - S^T k~);  S <- S + k~ u^T;  o = S^T q~
+
+    qkv float32 [n, .]: q of key head j at q_col + j * dim, k at k_col + j * dim, v of head h at v_col + h * E;
+    ab float32 [n, .]: b of head h at b_col + h, a at a_col + h; value head h reads key head h // (H / kv_heads).
+    out float32 [n, H * E]."""
+    n, wq, ld_qkv = _rows(qkv, "qkv")
+    na, wa, ld_ab = _rows(ab, "ab")
+    _need(qkv.dtype == torch.float32 and ab.dtype == torch.float32 and na == n, "the delta rule reads float32 rows")
+    _need(state.dim() == 4 and state.is_contiguous() and state.dtype == torch.float32, "state must be float32 [requests, H, E, Dk]")
+    H, E, Dk = state.shape[1:]
+    G, D = int(kv_heads), int(dim)
+    _need(G > 0 and H % G == 0 and 0 < D <= 256 and Dk == delta_key_extent(D), "the delta rule takes key sizes up to 256, H a multiple of the key heads")
+    _need(min(q_col, k_col, v_col, a_col, b_col) >= 0 and max(q_col, k_col) + G * D <= wq and v_col + H * E <= wq
+          and max(a_col, b_col) + H <= wa, "q, k, v, a or b exceed their rows")
+    no, wo, ldo = _rows(out, "out")
+    _need(no == n and wo == H * E and out.dtype == torch.float32, "out must be float32 [n, H * E]")
+    _need(A_log.numel() == H and dt_bias.numel() == H and A_log.dtype == torch.float32 and dt_bias.dtype == torch.float32,
+          "one float32 A_log and dt_bias per head")
+    _need(seq0 >= 0 and q_start.numel() >= seq0 + n_seqs + 1 and state_slots.numel() >= seq0 + n_seqs, "sequence metadata is too short")
+    check(library().tw_delta_rule(_dev(qkv), ld_qkv, int(q_col), int(k_col), int(v_col), _dev(ab), ld_ab, int(b_col), int(a_col),
+                                  _dev(A_log), _dev(dt_bias), _dev(state), _dev(q_start, torch.int32, "q_start"),
+                                  _dev(state_slots, torch.int32, "state_slots"), _dev(out), ldo, int(seq0), int(n_seqs),
+                                  H, G, D, E, Dk, float(q_scale), _stream()), "delta_rule")
+    return out
+
+
+def head_norm_gate(o, gate, weight, out, heads, value_dim, eps):
+    """out[n, h, e] = o[n, h, e] / sqrt(mean_e o^2 + eps) * weight[e] * silu(gate[n, h, e]); o and gate float32, weight
+    float32 [value_dim] shared by the heads, out of the compute type."""
+    n, wo, ld_o = _rows(o, "o")
+    ng, wg, ld_g = _rows(gate, "gate")
+    nn, wn, ld_n = _rows(out, "out")
+    _need(o.dtype == torch.float32 and gate.dtype == torch.float32, "o and gate are float32")
+    _need(ng == n and nn == n and min(wo, wg, wn) >= heads * value_dim and weight.numel() == value_dim, "head_norm_gate shapes do not agree")
+    check(library().tw_head_norm_gate(dtype_id(out.dtype), _dev(o), ld_o, _dev(gate), ld_g, _dev(weight, torch.float32, "weight"),
+                                      _dev(out), ld_n, n, int(heads), int(value_dim), float(eps), _stream()), "head_norm_gate")
+    return out
+
+
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(h, router, top, ids, weights):
+    """ids[n, top], weights[n, top]: per row of h the `top` experts with the largest router logits router @ h (float32
+    products of h's values as they are; the lowest index wins a tie), and the sigmoid of each chosen logit."""
+    n, C, ld_h = _rows(h, "h")
+    X = router.shape[0]
+    _need(router.dtype == torch.float32 and router.is_contiguous() and tuple(router.shape) == (X, C), "the router is float32 [experts, C]")
+    _need(0 < top <= X <= MOE_MAX_EXPERTS, f"1 to {MOE_MAX_EXPERTS} experts, of which at most all are chosen")
+    _need(ids.is_contiguous() and weights.is_contiguous() and tuple(ids.shape) == (n, top) and tuple(weights.shape) == (n, top),
+          "ids and weights are [n, top]")
+    check(library().tw_moe_route(dtype_id(h.dtype), _dev(h), ld_h, _dev(router), n, C, X, int(top), _dev(ids, torch.int32, "ids"),
+                                 _dev(weights, torch.float32, "weights"), _stream()), "moe_route")
+    return ids, weights
+
+
+def moe_capacity(items, experts):
+    """Rows the experts' order can take for ITEMS (token, choice) pairs: every expert's share rounded up to 16 rows."""
+    return int(library().tw_moe_capacity(int(items), int(experts)))
+
+
+def moe_pad(size):
+    """A size the grouped products take as their K: rounded up to a multiple of 32 (zeros fill the rest)."""
+    return (int(size) + 31) // 32 * 32
+
+
+def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch):
+    """x[n] += sum over a row's chosen experts e of down_e(glu(gate_e y, up_e y)), y = round(weights * h[n]), glu the
+    limited swish with LIMIT. gate, up [X, Fd, Cd], down [X, C, Fd] in h's type, zero padded (Fd, Cd: `moe_pad` of the
+    sizes). scratch(tag, shape, dtype) hands out the step's scratch tensors."""
+    n, C, ld_h = _rows(h, "h")
+    top = ids.shape[1]
+    X, Fd, Cd = gate.shape
+    _need(gate.is_contiguous() and up.is_contiguous() and down.is_contiguous() and gate.dtype == up.dtype == down.dtype == h.dtype,
+          "the experts' matrices are contiguous and of h's type")
+    _need(tuple(up.shape) == (X, Fd, Cd) and tuple(down.shape) == (X, C, Fd) and Cd == moe_pad(C) and Fd % 32 == 0,
+          "the experts' matrices are [X, Fd, Cd] and [X, C, Fd]")
+    _need(ids.is_contiguous() and weights.is_contiguous() and tuple(ids.shape) == (n, top) and tuple(weights.shape) == (n, top),
+          "ids and weights are [n, top]")
+    nx, cx, ld_x = _rows(x, "x")
+    _need(nx == n and cx == C and x.dtype == torch.float32, "x must be float32 [n, C]")
+    capacity = moe_capacity(n * top, X)
+    pos = scratch("moe.pos", (n * top,), torch.int32)
+    src_item = scratch("moe.src", (capacity,), torch.int32)
+    tile_expert = scratch("moe.tiles", (capacity // 16,), torch.int32)
+    xs = scratch("moe.xs", (capacity, Cd), h.dtype)
+    act = scratch("moe.act", (capacity, Fd), h.dtype)
+    ys = scratch("moe.ys", (capacity, C), torch.float32)
+    check(library().tw_moe_experts(dtype_id(h.dtype), _dev(h), ld_h, _dev(ids, torch.int32, "ids"),
+                                   _dev(weights, torch.float32, "weights"), n, top, X, _dev(gate), _dev(up), _dev(down), C, Cd, Fd,
+                                   float(limit), _dev(pos), _dev(src_item), _dev(tile_expert), _dev(xs), _dev(act), _dev(ys),
+                                   capacity, _dev(x), ld_x, _stream()), "moe_experts")
+    return x

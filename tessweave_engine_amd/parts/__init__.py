@@ -5,13 +5,15 @@ from .norms import RMSNorm
 from .positions import NoPositionEncoding, RotaryEmbedding
 from .attention import GroupedQueryAttention
 from .feedforward import GatedFeedForward, ReluSquaredFeedForward, SwiGLU
-from .blocks import DepthMixedBlock, PostNormBlock, PreNormBlock
+from .blocks import DepthMixedBlock, ParallelBlock, PostNormBlock, PreNormBlock
 from .embedding import HashedPairEmbedding, OutputHead, PositionedEmbedding, TokenEmbedding
 from .convolution import CausalConv
 from .parallel import GatedLinearRecurrence, MixedHeadAttention, MixerBranch, ParallelMixer
 from .side_input import SideTable, TokenSideInput
 from .latent import LatentAttention
 from .retention import Retention
+from .delta import GatedDeltaRule
+from .experts import RoutedExperts
 from .model import DecoderModel, walk
 
 __all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer", "Norm", "Part", "PositionEncoding",
@@ -20,4 +22,5 @@ __all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer",
            "JoinedLinear", "GatedFeedForward", "DepthMixedBlock", "PositionedEmbedding", "CausalConv",
            "GatedLinearRecurrence", "MixedHeadAttention", "MixerBranch", "ParallelMixer", "SideTable", "TokenSideInput",
            "HashedPairEmbedding", "LatentAttention", "PostNormBlock", "ReluSquaredFeedForward", "Retention",
+           "GatedDeltaRule", "ParallelBlock", "RoutedExperts",
            "DecoderModel", "walk"]

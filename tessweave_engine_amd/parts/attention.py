@@ -19,8 +19,14 @@ import torch
 
 class GroupedQueryAttention(Mixer):
     def __init__(self, prefix, hidden, q_heads, kv_heads, head_dim, position, qkv_bias=True,
-                 o_bias=False, window=None, scale=None, packed=True, head_hook=None, softcap=None):
-        """softcap: scaled scores pass through softcap * tanh(score / softcap) before the softmax (the attention
+                 o_bias=False, window=None, scale=None, packed=True, head_hook=None, softcap=None, value_dim=None,
+                 names=("q_proj", "k_proj", "v_proj", "o_proj"), suffixes=(".weight", ".bias")):
+        """value_dim: a value's size if it differs from a key's (head_dim). The kernels take one size for both: keys
+        and values are then both laid out with the larger of the two, tails of zeros (a key's zero tail adds nothing
+        to a score, a value's zero tail gives zero outputs, which meet zero columns of the output matrix).
+        names, suffixes: the checkpoint's names of the four matrices behind the prefix, and what follows a name
+        for its weight and its bias.
+        softcap: scaled scores pass through softcap * tanh(score / softcap) before the softmax (the attention
         kernels that take every type and page size then run; the fast bfloat16 ones have no such step).
         head_hook: an optional `HeadHook` that changes the projected q, k, v (bias added) in place before q
         and k are rotated: a per-head norm, a scaling. With a hook the projection is finished by its own
@@ -38,16 +44,20 @@ class GroupedQueryAttention(Mixer):
         # the result is exactly that of the unpadded head. `head_dim` is the size on the device from here on;
         # the scale and the rotation keep the checkpoint's size.
         self.checkpoint_head_dim = int(head_dim)
-        self.head_dim = (int(head_dim) + 15) // 16 * 16
+        self.value_dim = int(value_dim) if value_dim else int(head_dim)
+        if not 1 <= self.value_dim <= 256:
+            raise ValueError(f"the attention kernels take value sizes up to 256; value_dim {value_dim} is refused")
+        self.head_dim = (max(int(head_dim), self.value_dim) + 15) // 16 * 16
         pad = (self.checkpoint_head_dim, self.head_dim)
+        vpad = (self.value_dim, self.head_dim)
         self.position = position
         self.window = window
         self.scale = float(scale) if scale is not None else self.checkpoint_head_dim ** -0.5
         self.softcap = float(softcap) if softcap else 0.0
-        self.qkv = Linear([prefix + "q_proj", prefix + "k_proj", prefix + "v_proj"], hidden,
-                          [q_heads * head_dim, kv_heads * head_dim, kv_heads * head_dim], bias=qkv_bias, packed=packed,
-                          pad_out=pad)
-        self.o = Linear([prefix + "o_proj"], q_heads * head_dim, [hidden], bias=o_bias, pad_in=pad)
+        self.qkv = Linear([prefix + names[0], prefix + names[1], prefix + names[2]], hidden,
+                          [q_heads * head_dim, kv_heads * head_dim, kv_heads * self.value_dim], bias=qkv_bias, packed=packed,
+                          pad_out=[pad, pad, vpad], suffixes=suffixes)
+        self.o = Linear([prefix + names[3]], q_heads * self.value_dim, [hidden], bias=o_bias, pad_in=vpad, suffixes=suffixes)
         self.head_hook = head_hook
 
     def parts(self):

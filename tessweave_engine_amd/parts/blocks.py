@@ -43,6 +43,51 @@ def normalise(norm, ctx, x, pending=None, rows=None):
     return norm.forward(ctx, x, rows=rows)
 
 
+class ParallelBlock(Block):
+    """Mixer and feed-forward side by side, each behind a norm of its own, both of the same stream:
+
+        x <- x + mixer(norm1(x)) + ff(norm2(x))
+
+    mixer_norm, ffn_norm: `RMSNorm` parts (weights and eps; both norms are one kernel: the row is read and its
+    statistic formed once). ffn / ffn_norm may be None: the layer then has only the mixer. Both sublayers add into
+    the stream after both norms have read it. The sublayers' sums are complete when the block returns (a model of
+    such blocks is built with `defer_sums=False`)."""
+
+    def __init__(self, hidden, mixer_norm, mixer, ffn_norm=None, ffn=None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        if ffn_norm is not None and ffn_norm.eps != mixer_norm.eps:
+            raise ValueError("the two norms of a parallel block share their eps")
+        self.hidden = int(hidden)
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def tensor_specs(self):
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors, dtype, device):
+        for p in self.parts():
+            p.bind(tensors, dtype, device)
+
+    def forward(self, ctx, run, x, pending=None):
+        pending = fold_pending(x, pending)
+        n = ctx.n_tokens
+        h1 = ctx.scratch("norm.out", (n, self.hidden))
+        h2 = ctx.scratch("norm.out.second", (n, self.hidden)) if self.ffn is not None else None
+        ops.rmsnorm_pair(x, self.mixer_norm.weight, self.mixer_norm.eps, h1,
+                         self.ffn_norm.weight if self.ffn is not None else None, h2)
+        left = self.mixer.forward(ctx, run, h1, x)
+        if left is not None:
+            raise RuntimeError("a parallel block's mixer must add into the stream itself")
+        if self.ffn is not None:
+            left = self.ffn.forward(ctx, h2, x)
+            if left is not None:
+                raise RuntimeError("a parallel block's feed-forward must add into the stream itself")
+        return None
+
+
 class PostNormBlock(Block):
     """Norm after the sum, with an optional scale per channel on each sublayer's result:
 

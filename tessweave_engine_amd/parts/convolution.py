@@ -49,12 +49,13 @@ class CausalConv(Part):
     def state_need(self):
         return (self.state_name, FixedState((2, max(self.taps - 1, 1), self.channels), "float32"))
 
-    def forward(self, ctx, run, src, out=None, out32=None):
-        """src: float32 rows (with a norm: the residual stream) or rows of the compute type."""
+    def forward(self, ctx, run, src, out=None, out32=None, activation=None):
+        """src: float32 rows (with a norm: the residual stream) or rows of the compute type.
+        activation "silu": the result passes SiLU before it is written."""
         state = ctx.cache.states[run.cache_slot][self.state_name]
         scratch = ctx.scratch("conv.rows", (src.shape[0],), torch.float32) if self.norm is not None else None
         ops.causal_conv(src, self.weight, state, ctx.q_start, ctx.kv_len, ctx.state_slots, ctx.state_phase, ctx.n_seqs,
                         out=out, out32=out32, norm_weight=self.norm.weight if self.norm is not None else None,
                         eps=self.norm.eps if self.norm is not None else 0.0, bias=self.bias, identity=self.identity,
-                        row_scratch=scratch)
+                        row_scratch=scratch, activation=activation)
         return out if out is not None else out32

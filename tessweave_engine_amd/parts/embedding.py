@@ -114,10 +114,12 @@ class HashedPairEmbedding(TokenEmbedding):
 
 
 class OutputHead(Part):
-    def __init__(self, name, vocab, hidden, tied_to=None, suffix=".weight"):
+    def __init__(self, name, vocab, hidden, tied_to=None, suffix=".weight", scale=1.0):
+        """scale: a factor on the logits, applied to the float32 product."""
         self.name, self.vocab, self.hidden = name, int(vocab), int(hidden)
         self.suffix = suffix
         self.tied_to = tied_to
+        self.scale = float(scale)
         self.weight = None
 
     def tensor_specs(self):
@@ -144,4 +146,7 @@ class OutputHead(Part):
     def forward(self, ctx, h):
         # The logits live in a shared scratch buffer: they are valid until the next step.
         logits = ctx.workspace.get("logits", (h.shape[0], self.vocab), torch.float32)
-        return ops.linear(h, self.matrix(), logits)
+        ops.linear(h, self.matrix(), logits)
+        if self.scale != 1.0:
+            ops.scale_values(logits, self.scale)
+        return logits

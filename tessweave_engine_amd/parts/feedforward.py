@@ -54,12 +54,17 @@ class GatedFeedForward(FeedForward):
     into the residual stream.
     """
 
-    def __init__(self, names, hidden, intermediate, activation="gelu_tanh", out_scale=1.0, suffix=".weight"):
-        if activation != "gelu_tanh":
-            raise ValueError("GatedFeedForward computes gelu_tanh; SwiGLU is the SiLU part")
+    def __init__(self, names, hidden, intermediate, activation="gelu_tanh", out_scale=1.0, suffix=".weight", limit=None):
+        """activation: "gelu_tanh", "silu", or "swish_limited", which needs `limit` L and computes
+        g' * sigmoid(1.702 g') * (u' + 1) with g' = min(gate, L), u' = clamp(up, -L, L) (and takes no out_scale)."""
+        if activation not in ("gelu_tanh", "silu", "swish_limited"):
+            raise ValueError("GatedFeedForward computes gelu_tanh, silu or swish_limited")
+        if activation == "swish_limited" and (limit is None or not float(limit) > 0 or float(out_scale) != 1.0):
+            raise ValueError("swish_limited needs a positive limit and takes no out_scale")
         gate, up, down = names
         self.hidden, self.intermediate, self.out_scale = int(hidden), int(intermediate), float(out_scale)
         self.activation = activation
+        self.limit = float(limit) if limit is not None else None
         self.gate_up = Linear([gate, up], hidden, [intermediate, intermediate], glu=True, suffixes=(suffix, ".bias"))
         self.down = Linear([down], intermediate, [hidden], suffixes=(suffix, ".bias"))
 
@@ -76,12 +81,20 @@ class GatedFeedForward(FeedForward):
     def forward(self, ctx, h, x, accumulate=True):
         n = h.shape[0]
         act = ctx.scratch("ffn.act", (n, self.intermediate))
+        limited = self.activation == "swish_limited"
         if self.gate_up.gated:
-            self.gate_up.forward_glu(ctx, h, act, activation=self.activation, factor=self.out_scale)
+            self.gate_up.forward_glu(ctx, h, act, activation=self.activation, factor=self.limit if limited else self.out_scale)
         else:
             gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
             self.gate_up.forward(ctx, h, gu)
-            ops.gelu_mul(gu, act, self.out_scale)
+            if limited:
+                ops.swish_limited_mul(gu, act, self.limit)
+            elif self.activation == "silu" and self.out_scale == 1.0:
+                ops.silu_mul(gu, act)
+            elif self.activation == "silu":
+                raise ValueError("silu with an output scale needs an intermediate size that is a multiple of 16")
+            else:
+                ops.gelu_mul(gu, act, self.out_scale)
         self.down.forward(ctx, act, x, residual=x if accumulate else None)
         return None
 

@@ -15,8 +15,11 @@ def walk(part):
 
 
 class DecoderModel(Part):
-    def __init__(self, config, embedding, blocks, final_norm, head, schedule=None):
-        """SCHEDULE defaults to every block once, in order, each with its own cache slot."""
+    def __init__(self, config, embedding, blocks, final_norm, head, schedule=None, defer_sums=True):
+        """SCHEDULE defaults to every block once, in order, each with its own cache slot.
+        defer_sums=False: no part may leave split-K sums pending for a later norm (for arrangements whose blocks
+        do not take them), whatever the norms could fold."""
+        self.defer_sums = bool(defer_sums)
         self.config = config
         self.embedding = embedding
         self.blocks = list(blocks)
@@ -45,7 +48,7 @@ class DecoderModel(Part):
     @property
     def defers_sums(self):
         """May mixers and feed-forwards leave split-K sums to the next norm? Only if every norm folds them."""
-        return all(p.folds_pending for p in walk(self) if isinstance(p, Norm))
+        return self.defer_sums and all(p.folds_pending for p in walk(self) if isinstance(p, Norm))
 
     def tensor_specs(self):
         specs, seen = [], set()

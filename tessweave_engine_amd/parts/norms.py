@@ -7,14 +7,17 @@ float32 (exact for a bfloat16 checkpoint).
 from __future__ import annotations
 
 from ..kernels import ops
-from ..weights.spec import VECTOR, ONE_PLUS_NORMAL, TensorSpec
+from ..weights.spec import NORMAL, VECTOR, ONE_PLUS_NORMAL, TensorSpec
 from .base import Norm
 
 
 class RMSNorm(Norm):
     folds_pending = True
 
-    def __init__(self, name, size, eps, suffix=".weight"):
+    def __init__(self, name, size, eps, suffix=".weight", offset=0.0):
+        """offset: what the stored weight is to be increased by (1.0 for checkpoints that keep their norm weights
+        around zero, y = unit(x) * (1 + w)); the sum is formed once, in float32, when the weights are bound."""
+        self.offset = float(offset)
         self.name = name
         self.suffix = suffix              # what follows the name in the checkpoint
         self.size = int(size)
@@ -22,10 +25,12 @@ class RMSNorm(Norm):
         self.weight = None
 
     def tensor_specs(self):
-        return [TensorSpec(self.name + self.suffix, (self.size,), VECTOR, ONE_PLUS_NORMAL)]
+        return [TensorSpec(self.name + self.suffix, (self.size,), VECTOR, NORMAL if self.offset == 1.0 else ONE_PLUS_NORMAL)]
 
     def bind(self, tensors, dtype, device):
         self.weight = tensors.pop(self.name + self.suffix).contiguous()
+        if self.offset:
+            self.weight = (self.weight + self.offset).contiguous()
 
     def weight_tensors(self):
         return [self.weight]
