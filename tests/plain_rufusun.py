@@ -134,6 +134,15 @@ def routed_ffn(h, w, mlp):
     return out
 
 
+def router_margin(h, w, mlp):
+    """Per token: how far the last chosen expert's router logit lies above the best one not chosen (inf if all run)."""
+    top = mlp["router"]["top"]
+    z = torch.sort(h @ w["router"].T, -1, descending=True).values
+    if top >= z.shape[1]:
+        return torch.full((h.shape[0],), float("inf"), dtype=h.dtype)
+    return z[:, top - 1] - z[:, top]
+
+
 def sub(tensors, prefix):
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
@@ -148,15 +157,15 @@ def layer_order(config):
     return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
 
-def forward(config, tensors, tokens, keep_layers=False):
-    """Logits [T, V] of a whole sequence (and, with keep_layers, the stream after every layer run)."""
+def forward(config, tensors, tokens, keep_layers=False, margins=None):
+    """Logits [T, V] of a whole sequence (and, with keep_layers, the stream after every layer run). margins: a list
+    that receives, per run of a layer with routed experts, every token's `router_margin`."""
     eps = config["norm"]["eps"]
     x = tensors["embed"][torch.tensor([int(t) for t in tokens], dtype=torch.long)]
     kept = []
     for i in layer_order(config):
         layer, p = config["layers"][i], f"l{i}."
         h1 = offset_norm(x, tensors[p + "norm1"], eps)
-        h2 = offset_norm(x, tensors[p + "norm2"], eps)
         mix = sub(tensors, p + "mix.")
         if layer["type"] == "attention":
             y = capped_attention(h1, mix, layer["mixer"])
@@ -166,8 +175,11 @@ def forward(config, tensors, tokens, keep_layers=False):
             raise ValueError(layer["type"])
         mlp = layer.get("mlp")
         if mlp:
+            h2 = offset_norm(x, tensors[p + "norm2"], eps)        # of the same x as the mixer's norm
             w = sub(tensors, p + "mlp.")
             y = y + (dense_ffn(h2, w) if mlp["kind"] == "dense" else routed_ffn(h2, w, mlp))
+            if margins is not None and mlp["kind"] != "dense":
+                margins.append(router_margin(h2, w, mlp))
         x = x + y
         kept.append(x)
     logits = (offset_norm(x, tensors["final.norm"], eps) @ tensors["head"].T) * config["logit_scale"]
