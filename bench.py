@@ -19,7 +19,7 @@ as the weights; `prefill_32k_prompts`: tokens a second over those prompts, which
 go through in portions of 2,048); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
 (`gen512_b*`, decoded tokens a second over the generated part).
 
-Other sizes of the architecture: --shape 14b|32b. --design kanavik|dinutar measures that
+Other sizes of the architecture: --shape 14b|32b. --design kanavik|dinutar|rufusun measures that
 design's prefill and decode at a few layer sizes, each beside the Qwen2 decoder at equal
 width, heads, feed-forward and depth (one JSON line a size). --serve measures continuous
 batching under Poisson arrivals instead (prompts of 128..4,096 tokens, 256
@@ -89,7 +89,7 @@ def parse():
                    help="with --serve: the largest prompt portion in one step (larger: more prompt tokens a second and "
                         "a shorter time to the first token, longer steps for the requests that are decoding)")
     p.add_argument("--rate", type=float, default=16.0, help="mean arrivals a second (0: all at once)")
-    p.add_argument("--design", default="", choices=["", "kanavik", "dinutar"],
+    p.add_argument("--design", default="", choices=["", "kanavik", "dinutar", "rufusun"],
                    help="instead: prefill and decode throughput of another design at a few layer sizes (--design-sizes), "
                         "each beside the Qwen2 decoder at equal width, heads, feed-forward and depth; one JSON line a size")
     p.add_argument("--design-sizes", default="1b,3b,7b", help="which of the design's sizes to run, comma separated")
@@ -144,6 +144,30 @@ def dinutar_config(size, layers, context):
             "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": out}
 
 
+# The Rufusun design at those widths: layers in the order delta rule, delta rule, attention, attention, the second of each
+# pair with routed experts in place of the dense feed-forward (16 experts of a quarter of the dense inner size, two a
+# token, beside a shared expert of the same size: three quarters of the dense layer's arithmetic a token, four times
+# its weights). Delta rule: the size's heads as value heads of the head size, its key/value heads as key heads,
+# convolutions of four taps. Attention: rotation over half of a head, a soft cap of 30.
+def rufusun_config(size, layers, context):
+    width, heads, kv_heads, dim, ff, _ = DESIGN_SIZES[size]
+    dense = {"kind": "dense", "ff": ff}
+    routed = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ff // 4, "limit": 7.0},
+              "shared": {"ff": ff // 4, "limit": 7.0}}
+    out = []
+    for i in range(layers):
+        mlp = routed if i % 2 else dense
+        if i % 4 < 2:
+            out.append({"type": "delta", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4}})
+        else:
+            out.append({"type": "attention", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                  "softcap": 30.0, "rot": {"base": 1e6, "dims": dim // 2}}})
+    return {"architecture": "Rufusun", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "layers": out}
+
+
 def qwen2_config_like(size, layers, context):
     width, heads, kv_heads, dim, ff, _ = DESIGN_SIZES[size]
     return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
@@ -155,6 +179,7 @@ def design_run(args, torch):
     """One JSON line a size: the design's prefill and decode throughput and, beside it, the Qwen2 decoder's at equal
     width, heads, feed-forward size and depth (same engine, same scheduler, random weights)."""
     from tessweave_engine_amd.config import config_from_dict
+    from tessweave_engine_amd.parts import walk
     from tessweave_engine_amd.weights import random_model
     use_graphs = not args.no_graphs
     steps, warmup = min(args.steps, 64), min(args.warmup, 8)
@@ -163,13 +188,16 @@ def design_run(args, torch):
                 "sizes": dict(zip(("width", "heads", "kv_heads", "head_dim", "ff", "window"), DESIGN_SIZES[size])),
                 "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens,
                 "data": "synthetic: uniform-random token ids, random weights"}
-        make = {"kanavik": kanavik_config, "dinutar": dinutar_config}[args.design]
+        make = {"kanavik": kanavik_config, "dinutar": dinutar_config, "rufusun": rufusun_config}[args.design]
         models = [(args.design, make(size, args.design_layers, args.context))]
         if not args.design_only:
             models.append(("qwen2", qwen2_config_like(size, args.design_layers, args.context)))
         for name, cfg in models:
             model = random_model(config_from_dict(cfg), args.seed, dtype=args.dtype, device="cuda:0")
             entry = {"weight_gb": round(model.weight_bytes() / 1e9, 3)}
+            routed = sum(p.expert_bytes() * p.experts for p in walk(model) if hasattr(p, "expert_bytes"))
+            if routed:          # (not among the weights a step reads in full: a step reads the experts its tokens chose)
+                entry["routed_expert_gb"] = round(routed / 1e9, 3)
             if args.prefill_tokens > 0:
                 ms = prefill_run(model, torch, args.prefill_tokens, args.dtype, args.seed)
                 entry.update(prefill_ms=round(ms, 3), prefill_tokens_per_s=round(args.prefill_tokens / (ms / 1000), 1))

@@ -10,11 +10,13 @@
 // order from the request's state, which the same lanes read at the start and write at the end: nothing depends on
 // how a prompt was cut.
 //
-// A workgroup owns 64 value columns of one (sequence, head). A wave holds 16 of them: lane = 4 * column + slice,
-// and a lane keeps the quarter `slice` of its column of S in registers (DPL elements), so both products of a token
-// are DPL multiply-adds and two lane swaps inside a quad. The state lies in memory as [H][E][Dk] (a column of S is
-// contiguous), Dk = 4 * DPL. Tokens are staged in LDS in chunks: the waves share a chunk's tokens out, norm q and k,
-// form beta and g, then all walk the chunk.
+// A workgroup owns 256 / KS value columns of one (sequence, head). A wave holds 64 / KS of them: lane = KS * column +
+// slice, and a lane keeps part `slice` of its column of S in registers (DPL elements), so both products of a token are
+// DPL multiply-adds and a sum over KS neighbouring lanes (DPP: inside a quad, or rotations of a row of 16). What a token
+// costs is the length of that dependent chain, so keys longer than 16 are cut into 16 slices: 8 multiply-adds a
+// product at a key size of 128, and a head's columns spread over eight workgroups. The state lies in memory as
+// [H][E][Dk] (a column of S is contiguous), Dk <= KS * DPL. Tokens are staged in LDS in chunks: the waves share a
+// chunk's tokens out, norm q and k, form beta and g, then all walk the chunk.
 #include "tw_common.h"
 
 #define TW_DELTA_CHUNK 16
@@ -36,29 +38,38 @@ template <int CTRL>
 __device__ __forceinline__ float delta_quad_swap(float v) {
   return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
 }
-// sum over the four lanes of a quad; every lane gets it
-__device__ __forceinline__ float delta_quad_sum(float v) {
-  v += delta_quad_swap<0xB1>(v);      // lanes 1 0 3 2
-  v += delta_quad_swap<0x4E>(v);      // lanes 2 3 0 1
+// sum over KS neighbouring lanes (4: a quad; 16: a row); every lane gets it
+template <int KS>
+__device__ __forceinline__ float delta_group_sum(float v) {
+  if constexpr (KS == 4) {
+    v += delta_quad_swap<0xB1>(v);    // lanes 1 0 3 2
+    v += delta_quad_swap<0x4E>(v);    // lanes 2 3 0 1
+  } else {
+    v += delta_quad_swap<0x128>(v);   // the row rotated by 8 lanes, then by 4, 2, 1
+    v += delta_quad_swap<0x124>(v);
+    v += delta_quad_swap<0x122>(v);
+    v += delta_quad_swap<0x121>(v);
+  }
   return v;
 }
 
 __device__ __forceinline__ float delta_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
-template <int DPL>
+template <int DPL, int KS>
 __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) {
-  constexpr int SL = DPL + 4;                        // a slice's stride in LDS: the four slices of a quad meet different banks
-  constexpr int ROW = 4 * SL;
+  constexpr int SL = DPL + 4;                        // a slice's stride in LDS: the slices a read meets lie in different banks
+  constexpr int ROW = KS * SL;
+  constexpr int CW = 256 / KS, CV = 64 / KS;         // value columns a workgroup, a wave
   __shared__ __attribute__((aligned(16))) float q_s[TW_DELTA_CHUNK][ROW];
   __shared__ __attribute__((aligned(16))) float k_s[TW_DELTA_CHUNK][ROW];
-  __shared__ float v_s[TW_DELTA_CHUNK][64];
+  __shared__ float v_s[TW_DELTA_CHUNK][CW];
   __shared__ float gate_s[TW_DELTA_CHUNK][2];        // beta, g
-  const int blocks_e = (a.E + 63) / 64;
+  const int blocks_e = (a.E + CW - 1) / CW;
   const int eb = blockIdx.x % blocks_e, head = blockIdx.x / blocks_e;
   const int s = seq0 + blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int slice = lane & 3;
-  const int e = eb * 64 + wave * 16 + (lane >> 2);
+  const int slice = lane & (KS - 1);
+  const int e = eb * CW + wave * CV + lane / KS;
   const bool live = e < a.E;
   const int kh = head / (a.H / a.G);
   const int first = a.q_start[s], last = a.q_start[s + 1];
@@ -95,13 +106,13 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) 
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int d = lane + 64 * j;
-        if (d < 4 * DPL) {
+        if (d < KS * DPL) {
           q_s[i][(d / DPL) * SL + d % DPL] = qv[j] * qn;
           k_s[i][(d / DPL) * SL + d % DPL] = kv[j] * kn;
         }
       }
-      const int ev = eb * 64 + lane;
-      v_s[i][lane] = ev < a.E ? row[a.v_col + (size_t)head * a.E + ev] : 0.f;
+      const int ev = eb * CW + lane;
+      if (lane < CW) v_s[i][lane] = ev < a.E ? row[a.v_col + (size_t)head * a.E + ev] : 0.f;
       if (lane == 0) {
         const float* ab = a.ab + (size_t)(t0 + i) * a.ld_ab;
         const float b = ab[a.b_col + head], x = ab[a.a_col + head];
@@ -123,8 +134,8 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) 
         d2 = __fmaf_rn(S[j + 2], kq[2], d2);
         d3 = __fmaf_rn(S[j + 3], kq[3], d3);
       }
-      const float dot = delta_quad_sum((d0 + d1) + (d2 + d3));
-      const float u = beta * (v_s[i][wave * 16 + (lane >> 2)] - g * dot);
+      const float dot = delta_group_sum<KS>((d0 + d1) + (d2 + d3));
+      const float u = beta * (v_s[i][wave * CV + lane / KS] - g * dot);
       float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
       for (int j = 0; j < DPL; j += 4) {
@@ -139,7 +150,7 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) 
         o2 = __fmaf_rn(S[j + 2], qq[2], o2);
         o3 = __fmaf_rn(S[j + 3], qq[3], o3);
       }
-      const float o = delta_quad_sum((o0 + o1) + (o2 + o3));
+      const float o = delta_group_sum<KS>((o0 + o1) + (o2 + o3));
       if (live && slice == 0) a.out[(size_t)(t0 + i) * a.ld_out + (size_t)head * a.E + e] = o;
     }
   }
@@ -161,12 +172,14 @@ extern "C" int tw_delta_rule(const float* qkv, long ld_qkv, int q_col, int k_col
   if (n_seqs == 0) return 0;
   DeltaArgs a{qkv, ld_qkv, q_col, k_col, v_col, ab, ld_ab, b_col, a_col, A_log, dt_bias, state, q_start, state_slots,
               out, ld_out, H, G, D, E, Dk, q_scale};
-  const dim3 grid(H * tw_div_up(E, 64), n_seqs);
-  if (Dk <= 16) delta_walk_kernel<4><<<grid, 256, 0, stream>>>(a, seq0);
-  else if (Dk <= 32) delta_walk_kernel<8><<<grid, 256, 0, stream>>>(a, seq0);
-  else if (Dk <= 64) delta_walk_kernel<16><<<grid, 256, 0, stream>>>(a, seq0);
-  else if (Dk <= 128) delta_walk_kernel<32><<<grid, 256, 0, stream>>>(a, seq0);
-  else delta_walk_kernel<64><<<grid, 256, 0, stream>>>(a, seq0);
+  if (Dk <= 16) {
+    delta_walk_kernel<4, 4><<<dim3(H * tw_div_up(E, 64), n_seqs), 256, 0, stream>>>(a, seq0);
+  } else {
+    const dim3 grid(H * tw_div_up(E, 16), n_seqs);
+    if (Dk <= 64) delta_walk_kernel<4, 16><<<grid, 256, 0, stream>>>(a, seq0);
+    else if (Dk <= 128) delta_walk_kernel<8, 16><<<grid, 256, 0, stream>>>(a, seq0);
+    else delta_walk_kernel<16, 16><<<grid, 256, 0, stream>>>(a, seq0);
+  }
   return TW_LAUNCH_RESULT();
 }
 
