@@ -34,6 +34,14 @@ template <typename T> struct KeyQuad;          // 4 consecutive keys of one d (A
 template <> struct KeyQuad<float> { typedef f32x4 Type; };
 template <> struct KeyQuad<bf16_t> { typedef bf16x4 Type; };
 
+// softcap * tanh(x / softcap) of a raw score x (before the scale): tanh(y) = 1 - 2 / (e^(2y) + 1), with the hardware's
+// exponential and reciprocal (both exact to a unit in the last place; the result is off by less than 1e-6 of the cap).
+// cap_raw = softcap / scale, two_over = 2 * log2(e) * scale / softcap: the result is again a raw score.
+__device__ __forceinline__ float tw_softcap_raw(float x, float cap_raw, float two_over) {
+  const float t = __builtin_amdgcn_exp2f(x * two_over);
+  return fmaf(-2.f * cap_raw, __builtin_amdgcn_rcpf(t + 1.f), cap_raw);
+}
+
 template <typename T, int DTMAX> struct AttnShape {
   static constexpr int EPF = Elem<T>::kPerFrag;
   static constexpr int NSMAX = (DTMAX * 16 / EPF + 3) / 4;    // MFMA steps over head_dim
@@ -55,8 +63,7 @@ struct AttnArgs {
   float* part_ml;         // [seq - seq0][q_heads][splits][2]  (max, sum)
   int q_heads, kv_heads, head_dim, page_size, window;
   float scale;
-  float softcap;          // > 0: scores (after the scale) pass through softcap * tanh(score / softcap); the kernels
-                          // that take every type and page size only
+  float softcap;          // > 0: scores (after the scale) pass through softcap * tanh(score / softcap)
   int splits;
   int page_shift;         // log2(page_size) if it is a power of two, else -1
   int n_seqs, max_tiles;  // prefill (bfloat16 kernel): sequences of the launch, row tiles of the longest
@@ -280,7 +287,7 @@ struct KVBlock {
 
 template <bool V> struct BoolTag { static constexpr bool value = V; };
 
-template <int DTMAX, bool EXACT>
+template <int DTMAX, bool EXACT, bool CAP = false>
 __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
   constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
   __shared__ __attribute__((aligned(16))) float lds_o[3][16][DTMAX * 16 + 8];   // (rows of 32 bytes more than a multiple of 256: see tw_lds_swz4)
@@ -390,7 +397,9 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int p = p0 + 8 * g + e;
-      pr[e] = (!EDGE || (p < kv_len && p >= lo)) ? s[e >> 2][e & 3] * a.scale : -INFINITY;
+      float sc = s[e >> 2][e & 3];
+      if constexpr (CAP) sc = tw_softcap_raw(sc, a.softcap / a.scale, 2.88539008177792681472f * a.scale / a.softcap);
+      pr[e] = (!EDGE || (p < kv_len && p >= lo)) ? sc * a.scale : -INFINITY;
       mx = fmaxf(mx, pr[e]);
     }
     mx = tw_rows_max(mx);
@@ -633,7 +642,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 
 // EXACT: head_dim == 16 * DTMAX, so every loop over the head has compile-time bounds (with run-time
 // bounds the compiler indexes the accumulators dynamically, several instructions per MFMA).
-template <int DTMAX, bool EXACT, int RT>
+template <int DTMAX, bool EXACT, int RT, bool CAP = false>
 __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   constexpr int TR = 64 * RT;                           // rows of a workgroup's tile: RT tiles of 16 per wave
   constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
@@ -699,6 +708,9 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const int first_pos = kv_len - q_len;
   const bool whole_chunks = EXACT || (chunks & 3) == 0;  // head_dim a multiple of 32: no partial MFMA step
   const float c2 = a.scale * 1.44269504088896340736f;    // scores are kept in the log2 domain
+  // With a soft cap the raw scores are replaced by capped raw scores as soon as they leave the matrix unit
+  // (cap / scale * tanh(raw * scale / cap)): everything after that is the same arithmetic.
+  const float cap_raw = CAP ? a.softcap / a.scale : 0.f, cap_two_over = CAP ? 2.f * c2 / a.softcap : 0.f;
 
   // ---- this wave's two row tiles -----------------------------------------------
   bf16x8 qf[RT][NSMAX];
@@ -909,6 +921,12 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     k_fragments(buf, kf);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) scores_of(rt, kf, s);
+    if constexpr (CAP) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[rt][e >> 2][e & 3] = tw_softcap_raw(s[rt][e >> 2][e & 3], cap_raw, cap_two_over);
+    }
     if (edge) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
@@ -1044,6 +1062,13 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       bf16x8 pb;
       probabilities(rt, s, pb);
       products(rt, vf, pb);
+    }
+    if constexpr (CAP) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          s_next[rt][e >> 2][e & 3] = tw_softcap_raw(s_next[rt][e >> 2][e & 3], cap_raw, cap_two_over);
     }
 #pragma unroll
     for (int i = 0; i < 2 * NSMAX * RT; ++i) {
@@ -1258,7 +1283,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     reference(s_now);
   }
   run_to(both_begin, step_by_step);
-  if constexpr (EXACT && PIPELINED) {
+  if constexpr (EXACT && PIPELINED && !CAP) {          // (the iteration ordered by hand has no slot for a cap's arithmetic)
     // (blk_end - 1 is the only block of the workgroup that may cross the end of the sequence)
     const bool all_whole = blk_end * 32 <= kv_len;
     const int ordered_end = all_whole ? both_end : min(both_end, blk_end - 5);
@@ -1414,8 +1439,8 @@ extern "C" long tw_attn_prefill_workspace_floats(int n_tokens, int q_heads, int 
   return max_chunks > 1 ? (long)n_tokens * q_heads * max_chunks * (head_dim + 2) : 0;
 }
 
-template <int DTMAX, bool EXACT>
-static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
+template <int DTMAX, bool EXACT, bool CAP>
+static int prefill_bf16_launch_as(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
   const int G = a.q_heads / a.kv_heads;
   const long rows = (long)max_q_len * G;
   a.n_seqs = n_seqs;
@@ -1428,22 +1453,28 @@ static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_
   const size_t lds_bytes = TW_PF_STAGES * (32 * (DTMAX * 32 + 32) + DTMAX * 16 * TW_PF_VROW);
   static bool attribute_set = false;
   if (!attribute_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<DTMAX, EXACT, 1>,
+    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<DTMAX, EXACT, 1, CAP>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<DTMAX, EXACT, 2>,
+      e = hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<DTMAX, EXACT, 2, CAP>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     attribute_set = true;
   }
   if (a.tile_rows == 64)
-    attn_prefill_bf16_kernel<DTMAX, EXACT, 1><<<grid, 256, lds_bytes, stream>>>(a);
+    attn_prefill_bf16_kernel<DTMAX, EXACT, 1, CAP><<<grid, 256, lds_bytes, stream>>>(a);
   else
-    attn_prefill_bf16_kernel<DTMAX, EXACT, 2><<<grid, 256, lds_bytes, stream>>>(a);
+    attn_prefill_bf16_kernel<DTMAX, EXACT, 2, CAP><<<grid, 256, lds_bytes, stream>>>(a);
   int err = TW_LAUNCH_RESULT();
   if (err || a.max_chunks <= 1) return err;
   attn_prefill_merge_kernel<<<dim3((unsigned)tw_div_up(rows, TW_MERGE_ROWS), a.kv_heads, n_seqs), 256, 0, stream>>>(a);
   return TW_LAUNCH_RESULT();
+}
+
+template <int DTMAX, bool EXACT>
+static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
+  if (a.softcap > 0.f) return prefill_bf16_launch_as<DTMAX, EXACT, true>(a, n_seqs, max_q_len, stream);
+  return prefill_bf16_launch_as<DTMAX, EXACT, false>(a, n_seqs, max_q_len, stream);
 }
 
 // =====================================================================================
@@ -1493,18 +1524,19 @@ static int decode_launch(AttnArgs a, int n_seqs, int generic, hipStream_t stream
   const int G = a.q_heads / a.kv_heads;
   dim3 grid(a.splits, a.kv_heads * ((G + 15) / 16), n_seqs);
   if (IsBf16<T>::value && a.page_shift >= 3 && !generic) {
-    if (a.head_dim == 64)
-      attn_decode_bf16_kernel<4, true><<<grid, 256, 0, stream>>>(a);
-    else if (a.head_dim < 64)
-      attn_decode_bf16_kernel<4, false><<<grid, 256, 0, stream>>>(a);
-    else if (a.head_dim == 128)
-      attn_decode_bf16_kernel<8, true><<<grid, 256, 0, stream>>>(a);
-    else if (a.head_dim < 128)
-      attn_decode_bf16_kernel<8, false><<<grid, 256, 0, stream>>>(a);
-    else if (a.head_dim == 256)
-      attn_decode_bf16_kernel<16, true><<<grid, 256, 0, stream>>>(a);
-    else
-      attn_decode_bf16_kernel<16, false><<<grid, 256, 0, stream>>>(a);
+    const bool cap = a.softcap > 0.f;
+#define TW_DECODE_CASE(DT, EX)                                                        \
+    do {                                                                              \
+      if (cap) attn_decode_bf16_kernel<DT, EX, true><<<grid, 256, 0, stream>>>(a);    \
+      else attn_decode_bf16_kernel<DT, EX, false><<<grid, 256, 0, stream>>>(a);       \
+    } while (0)
+    if (a.head_dim == 64) TW_DECODE_CASE(4, true);
+    else if (a.head_dim < 64) TW_DECODE_CASE(4, false);
+    else if (a.head_dim == 128) TW_DECODE_CASE(8, true);
+    else if (a.head_dim < 128) TW_DECODE_CASE(8, false);
+    else if (a.head_dim == 256) TW_DECODE_CASE(16, true);
+    else TW_DECODE_CASE(16, false);
+#undef TW_DECODE_CASE
   } else if (a.head_dim <= 64)
     attn_decode_kernel<T, 4><<<grid, 256, 0, stream>>>(a);
   else if (a.head_dim <= 128)
@@ -1534,7 +1566,6 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = splits;
   TW_REQUIRE(softcap >= 0.f);
   a.softcap = softcap;
-  if (softcap > 0.f) generic = 1;
   a.part_o = nullptr; a.part_ml = nullptr;
   a.page_shift = -1;
   for (int sh = 0; sh < 20; ++sh)
@@ -1592,7 +1623,6 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = 1;
   TW_REQUIRE(softcap >= 0.f);
   a.softcap = softcap;
-  if (softcap > 0.f) generic = 1;
   a.part_o = nullptr; a.part_ml = nullptr;
   a.max_chunks = 1; a.kv_chunk = 0;
   a.page_shift = -1;

@@ -17,6 +17,8 @@
 
 #define TW_MOE_MAX_EXPERTS 1024
 #define TW_MOE_TILE 16
+#define TW_MOE_WIDE 4                 /* tiles a workgroup takes at once in steps of many rows */
+#define TW_MOE_SPLITK_TILES 64        /* up to this many tiles a step, the waves of a workgroup split K */
 
 // ---- route ---------------------------------------------------------------------------------------------------
 template <typename T>
@@ -26,12 +28,40 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
   __shared__ float z[TW_MOE_MAX_EXPERTS];
   const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* x = h + (size_t)row * ld_h;
-  for (int e = wave; e < X; e += 4) {
-    const float* w = router + (size_t)e * C;
-    float sum = 0.f;
-    for (int c = lane; c < C; c += 64) sum = __fmaf_rn(w[c], tw_to_float(x[c]), sum);
-    sum = tw_wave_sum(sum);
-    if (lane == 0) z[e] = sum;
+  // A wave forms two experts' logits at a time, four elements a lane and load, eight loads in flight before the first
+  // is used: a logit is a chain of loads from memory, and their latency is all it costs.
+  const bool vec = C % 4 == 0 && ld_h % 4 == 0 && ((uintptr_t)h % 16 == 0) && ((uintptr_t)router % 16 == 0);
+  for (int e = 2 * wave; e < X; e += 8) {
+    const float* w0 = router + (size_t)e * C;
+    const float* w1 = router + (size_t)min(e + 1, X - 1) * C;
+    float s0 = 0.f, s1 = 0.f;
+    if (vec) {
+#pragma unroll 4
+      for (int c = 4 * lane; c < C; c += 256) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(w0 + c);
+        const f32x4 b = *reinterpret_cast<const f32x4*>(w1 + c);
+        float xv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xv[j] = tw_to_float(x[c + j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          s0 = __fmaf_rn(a[j], xv[j], s0);
+          s1 = __fmaf_rn(b[j], xv[j], s1);
+        }
+      }
+    } else {
+      for (int c = lane; c < C; c += 64) {
+        const float xv = tw_to_float(x[c]);
+        s0 = __fmaf_rn(w0[c], xv, s0);
+        s1 = __fmaf_rn(w1[c], xv, s1);
+      }
+    }
+    s0 = tw_wave_sum(s0);
+    s1 = tw_wave_sum(s1);
+    if (lane == 0) {
+      z[e] = s0;
+      if (e + 1 < X) z[e + 1] = s1;
+    }
   }
   __syncthreads();
   if (wave != 0) return;
@@ -78,7 +108,7 @@ extern "C" int tw_moe_route(int dtype, const void* h, long ld_h, const float* ro
 // every row is computed for itself and a token adds its rows in the order of its choices.
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ ids, int items, int X, int* __restrict__ pos,
                                                         int* __restrict__ src_item, int* __restrict__ tile_expert,
-                                                        int capacity, int tiles) {
+                                                        int capacity, int tiles, int unit) {
   __shared__ int count[TW_MOE_MAX_EXPERTS];
   __shared__ int offset[TW_MOE_MAX_EXPERTS + 1];
   for (int e = threadIdx.x; e < X; e += blockDim.x) count[e] = 0;
@@ -91,7 +121,7 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
     int at = 0;
     for (int e = 0; e < X; ++e) {
       offset[e] = at;
-      at += (count[e] + TW_MOE_TILE - 1) / TW_MOE_TILE * TW_MOE_TILE;
+      at += (count[e] + unit - 1) / unit * unit;
     }
     offset[X] = at;
   }
@@ -105,9 +135,14 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
   }
 }
 
+// The rows an expert's share is padded to: one tile, or, once the experts have a tile's rows each on average, the
+// TW_MOE_WIDE tiles that one workgroup of the grouped products then takes against one read of the expert's matrices.
+static int moe_unit(long items, int X) { return items >= (long)TW_MOE_TILE * X ? TW_MOE_TILE * TW_MOE_WIDE : TW_MOE_TILE; }
+
 extern "C" long tw_moe_capacity(long items, int X) {
-  // rows the experts' order can take: every expert's share rounded up to whole tiles
-  return (items + (long)X * (TW_MOE_TILE - 1) + TW_MOE_TILE - 1) / TW_MOE_TILE * TW_MOE_TILE;
+  // rows the experts' order can take: every expert's share rounded up to whole units (never fewer for more items)
+  const long unit = moe_unit(items, X);
+  return (items + (long)X * (unit - 1) + unit - 1) / unit * unit;
 }
 
 extern "C" int tw_moe_plan(const int* ids, int items, int X, int* pos, int* src_item, int* tile_expert, int capacity,
@@ -115,7 +150,8 @@ extern "C" int tw_moe_plan(const int* ids, int items, int X, int* pos, int* src_
   TW_REQUIRE(ids && pos && src_item && tile_expert && items >= 0 && X > 0 && X <= TW_MOE_MAX_EXPERTS);
   TW_REQUIRE(capacity >= tw_moe_capacity(items, X) && capacity % TW_MOE_TILE == 0);
   if (items == 0) return 0;
-  moe_plan_kernel<<<1, 1024, 0, stream>>>(ids, items, X, pos, src_item, tile_expert, capacity, capacity / TW_MOE_TILE);
+  moe_plan_kernel<<<1, 1024, 0, stream>>>(ids, items, X, pos, src_item, tile_expert, capacity, capacity / TW_MOE_TILE,
+                                          moe_unit(items, X));
   return TW_LAUNCH_RESULT();
 }
 
@@ -141,18 +177,27 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const T* __restrict__ h
 // One workgroup: a tile of 16 rows against 4 waves x NT x 16 columns of its expert's matrix W[ex] ([N][K], K a multiple
 // of 32). GLU: W and W2 are gate and up, the result glu(gate, up) goes out in the compute type; otherwise the float32
 // product. Operands go from memory straight into fragments (lane = 16 * piece + row reads 16 bytes).
-template <typename T, bool GLU, int NT>
+// SPLITK (steps of few rows, where the tiles in use are too few to fill the chip and every one streams its expert's whole
+// matrix): the four waves share one range of NT x 16 columns and take every fourth step over K each; their sums meet in
+// LDS and are added in the order of the waves.
+// MT > 1 (steps of many rows, whose experts' shares are padded to MT tiles): a workgroup takes MT tiles of one expert
+// against every fragment of the expert's matrices it reads.
+template <int N> struct MoeCount { static constexpr int value = N; };
+template <typename T, bool GLU, int NT, bool SPLITK = false, int MT = 1>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ A, long lda, const T* __restrict__ W,
                                                           const T* __restrict__ W2, const int* __restrict__ tile_expert,
                                                           void* __restrict__ out, long ldo, int N, int K, float limit) {
   constexpr int EPF = Elem<T>::kPerFrag;
-  const int tile = blockIdx.x;
+  const int tile = blockIdx.x * MT;
   const int ex = tile_expert[tile];
   if (ex < 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int col0 = (blockIdx.y * 4 + wave) * 16 * NT;
+  const int col0 = (SPLITK ? blockIdx.y : blockIdx.y * 4 + wave) * 16 * NT;
   if (col0 >= N) return;
+  constexpr int KSTEP = 4 * EPF;
+  constexpr int k_stride = SPLITK ? 4 * KSTEP : KSTEP;
+  const int k_first = SPLITK ? wave * KSTEP : 0;
   const T* a_ptr = A + (size_t)(tile * TW_MOE_TILE + r) * lda + g * EPF;
   const T* w_ptr[NT];
   const T* w2_ptr[NT];
@@ -162,35 +207,72 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
     w_ptr[t] = W + ((size_t)ex * N + col) * K + g * EPF;
     w2_ptr[t] = GLU ? W2 + ((size_t)ex * N + col) * K + g * EPF : nullptr;
   }
-  f32x4 acc[NT], acc2[NT];
+  f32x4 acc[MT][NT], acc2[MT][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = acc2[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-  for (int k = 0; k < K; k += 4 * EPF) {
-    const typename Elem<T>::Frag a = tw_load_frag(a_ptr + k);
-    typename Elem<T>::Frag b[NT], b2[NT];
+  for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      b[t] = tw_load_frag(w_ptr[t] + k);
-      if (GLU) b2[t] = tw_load_frag(w2_ptr[t] + k);
+    for (int t = 0; t < NT; ++t) acc[m][t] = acc2[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // U steps' operands are on their way before the first is used: what bounds this loop is the latency of memory
+  auto steps = [&](int k, auto count) {
+    constexpr int U = decltype(count)::value;
+    typename Elem<T>::Frag a[U][MT], b[U][NT], b2[U][NT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int m = 0; m < MT; ++m) a[u][m] = tw_load_frag(a_ptr + (size_t)m * TW_MOE_TILE * lda + k + u * k_stride);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        b[u][t] = tw_load_frag(w_ptr[t] + k + u * k_stride);
+        if (GLU) b2[u][t] = tw_load_frag(w2_ptr[t] + k + u * k_stride);
+      }
     }
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      tw_mma16(acc[t], a, b[t]);
-      if (GLU) tw_mma16(acc2[t], a, b2[t]);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          tw_mma16(acc[m][t], a[u][m], b[u][t]);
+          if (GLU) tw_mma16(acc2[m][t], a[u][m], b2[u][t]);
+        }
+  };
+  constexpr int U = MT > 1 ? 2 : GLU ? 4 : (NT > 2 ? 4 : 8);
+  int k = k_first;
+  for (; k + (U - 1) * k_stride < K; k += U * k_stride) steps(k, MoeCount<U>());
+  for (; k < K; k += k_stride) steps(k, MoeCount<1>());
+  static_assert(!SPLITK || MT == 1);
+  if constexpr (SPLITK) {
+    __shared__ f32x4 part[GLU ? 2 : 1][3][NT][64];
+    if (wave > 0) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        part[0][wave - 1][t][lane] = acc[0][t];
+        if (GLU) part[GLU ? 1 : 0][wave - 1][t][lane] = acc2[0][t];
+      }
     }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        acc[0][t] += part[0][w][t][lane];
+        if (GLU) acc2[0][t] += part[GLU ? 1 : 0][w][t][lane];
+      }
   }
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int col = col0 + t * 16 + r;
-    if (col >= N) continue;
+  for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const size_t at = (size_t)(tile * TW_MOE_TILE + 4 * g + j) * ldo + col;
-      if (GLU) ((T*)out)[at] = tw_from_float<T>(tw_swish_limited(acc[t][j], acc2[t][j], limit));
-      else ((float*)out)[at] = acc[t][j];
+    for (int t = 0; t < NT; ++t) {
+      const int col = col0 + t * 16 + r;
+      if (col >= N) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const size_t at = (size_t)((tile + m) * TW_MOE_TILE + 4 * g + j) * ldo + col;
+        if (GLU) ((T*)out)[at] = tw_from_float<T>(tw_swish_limited(acc[m][t][j], acc2[m][t][j], limit));
+        else ((float*)out)[at] = acc[m][t][j];
+      }
     }
-  }
 }
 
 // ---- combine: x[token] += its experts' rows, in the order of its choices ------------------------------------------
@@ -220,20 +302,50 @@ extern "C" int tw_moe_experts(int dtype, const void* h, long ld_h, const int* id
   if (code) return code;
   const int tiles = capacity / TW_MOE_TILE;
   const dim3 glu_grid(tiles, tw_div_up(Fd, 4 * 16 * 2)), down_grid(tiles, tw_div_up(C, 4 * 16 * 4));
+  // few rows: most tiles hold one or two rows and each streams its expert's matrices once; the waves then split K
+  const bool few = tiles <= TW_MOE_SPLITK_TILES;
+  const dim3 glu_few(tiles, tw_div_up(Fd, 16 * 2)), down_few(tiles, tw_div_up(C, 16 * 2));
+  const bool wide = moe_unit((long)n * top, X) == TW_MOE_TILE * TW_MOE_WIDE;
+  TW_REQUIRE(!wide || capacity % (TW_MOE_TILE * TW_MOE_WIDE) == 0);
+  const dim3 glu_wide(tiles / TW_MOE_WIDE, tw_div_up(Fd, 4 * 16 * 2)), down_wide(tiles / TW_MOE_WIDE, tw_div_up(C, 4 * 16 * 2));
   if (dtype == TW_DTYPE_BF16) {
     typedef bf16_t T;
     moe_gather_kernel<T><<<capacity, 256, 0, stream>>>((const T*)h, ld_h, weights, src_item, tile_expert, (T*)xs, C, Cd, top);
-    moe_grouped_kernel<T, true, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert,
-                                                                 act, Fd, Fd, Cd, limit);
-    moe_grouped_kernel<T, false, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr, tile_expert,
-                                                                  ys, C, C, Fd, 0.f);
+    if (few) {
+      moe_grouped_kernel<T, true, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                        tile_expert, act, Fd, Fd, Cd, limit);
+      moe_grouped_kernel<T, false, 2, true><<<down_few, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+                                                                         tile_expert, ys, C, C, Fd, 0.f);
+    } else if (wide) {
+      moe_grouped_kernel<T, true, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
+          (const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert, act, Fd, Fd, Cd, limit);
+      moe_grouped_kernel<T, false, 2, false, TW_MOE_WIDE><<<down_wide, 256, 0, stream>>>(
+          (const T*)act, Fd, (const T*)down, nullptr, tile_expert, ys, C, C, Fd, 0.f);
+    } else {
+      moe_grouped_kernel<T, true, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                   tile_expert, act, Fd, Fd, Cd, limit);
+      moe_grouped_kernel<T, false, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+                                                                    tile_expert, ys, C, C, Fd, 0.f);
+    }
   } else if (dtype == TW_DTYPE_F32) {
     typedef float T;
     moe_gather_kernel<T><<<capacity, 256, 0, stream>>>((const T*)h, ld_h, weights, src_item, tile_expert, (T*)xs, C, Cd, top);
-    moe_grouped_kernel<T, true, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert,
-                                                                 act, Fd, Fd, Cd, limit);
-    moe_grouped_kernel<T, false, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr, tile_expert,
-                                                                  ys, C, C, Fd, 0.f);
+    if (few) {
+      moe_grouped_kernel<T, true, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                        tile_expert, act, Fd, Fd, Cd, limit);
+      moe_grouped_kernel<T, false, 2, true><<<down_few, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+                                                                         tile_expert, ys, C, C, Fd, 0.f);
+    } else if (wide) {
+      moe_grouped_kernel<T, true, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
+          (const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert, act, Fd, Fd, Cd, limit);
+      moe_grouped_kernel<T, false, 2, false, TW_MOE_WIDE><<<down_wide, 256, 0, stream>>>(
+          (const T*)act, Fd, (const T*)down, nullptr, tile_expert, ys, C, C, Fd, 0.f);
+    } else {
+      moe_grouped_kernel<T, true, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                   tile_expert, act, Fd, Fd, Cd, limit);
+      moe_grouped_kernel<T, false, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+                                                                    tile_expert, ys, C, C, Fd, 0.f);
+    }
   } else {
     return TW_ERR_BAD_ARGUMENT;
   }

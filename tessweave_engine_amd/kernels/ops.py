@@ -399,7 +399,7 @@ def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out
 
     generic=True forces the kernel that takes every type and page size (bfloat16 with
     pages of a multiple of 8 keys otherwise runs a faster kernel of its own). softcap > 0 passes the scaled
-    scores through softcap * tanh(score / softcap) (that kernel only).
+    scores through softcap * tanh(score / softcap).
     """
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")

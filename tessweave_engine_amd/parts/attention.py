@@ -26,8 +26,7 @@ class GroupedQueryAttention(Mixer):
         to a score, a value's zero tail gives zero outputs, which meet zero columns of the output matrix).
         names, suffixes: the checkpoint's names of the four matrices behind the prefix, and what follows a name
         for its weight and its bias.
-        softcap: scaled scores pass through softcap * tanh(score / softcap) before the softmax (the attention
-        kernels that take every type and page size then run; the fast bfloat16 ones have no such step).
+        softcap: scaled scores pass through softcap * tanh(score / softcap) before the softmax.
         head_hook: an optional `HeadHook` that changes the projected q, k, v (bias added) in place before q
         and k are rotated: a per-head norm, a scaling. With a hook the projection is finished by its own
         kernel first (without one, few-row steps leave its split-K sums to the kernel that adds the bias,
