@@ -20,6 +20,7 @@
 #include "tw_common.h"
 
 #define TW_DELTA_CHUNK 16
+#define TW_DELTA_WALK_MOST 4          /* up to this many tokens a sequence, a step walks them one by one */
 
 struct DeltaArgs {
   const float* qkv; long ld_qkv;      // q of key head j at q_col + j * D, k at k_col + j * D, v of head h at v_col + h * E
@@ -159,12 +160,234 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) 
     if (held && slice * DPL + i < a.Dk) *reinterpret_cast<f32x4*>(S_mem + i) = f32x4{S[i], S[i + 1], S[i + 2], S[i + 3]};
 }
 
+// ---- many tokens a sequence: chunks of 16 tokens, each solved at once ----------------------------------------------
+// Inside a chunk with state S0 at its start, L_i = sum_{m <= i} log g_m (so that G_i = exp(L_i) and every quotient
+// G_i / G_j, j <= i, is an exponential of a sum of logarithms that are at most 0):
+//   u_i = beta_i (v_i - G_i S0^T k_i) - sum_{j < i} A_ij u_j,      A_ij = beta_i (G_i / G_j) (k_i . k_j)
+//   o_i = G_i S0^T q_i + sum_{j <= i} (G_i / G_j) (q_i . k_j) u_j
+//   S   = G_last S0 + sum_j (G_last / G_j) k_j u_j^T
+// which is the token-by-token rule written out. The products with S0 of all 16 tokens are independent of each other
+// (the walk's are a chain), the triangular system is solved by substitution per value column (after u_j is final every
+// later row takes its term off: one multiply-add deep a token), and the state is read and written once a chunk.
+// Lanes as in the walk with 16 slices: lane = 16 * column + slice; a workgroup owns 16 value columns of one (sequence,
+// head); thread 16 i + j also forms the pair (i, j) of A and of the read-out's matrix. Tokens behind a sequence's end
+// are staged as zeros with beta = 0 and g = 1: they change nothing. The next chunk's rows are on their way from memory
+// while this one is worked on.
+template <int DPL>
+__global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0) {
+  constexpr int KS = 16, C = 16, SL = DPL + 4;
+  constexpr int ROW = KS * SL + 4;                   // (+ 4: the 16 rows a read of the pair products meets lie in different banks)
+  constexpr int PW = C + 4;
+  __shared__ __attribute__((aligned(16))) float q_s[C][ROW];
+  __shared__ __attribute__((aligned(16))) float k_s[C][ROW];
+  __shared__ __attribute__((aligned(16))) float v_s[C][16];
+  __shared__ __attribute__((aligned(16))) float at_s[C][PW];     // at_s[j][i] = A_ij (0 unless j < i)
+  __shared__ __attribute__((aligned(16))) float qk_s[C][PW];     // qk_s[i][j] = (G_i / G_j) (q_i . k_j) (0 unless j <= i)
+  __shared__ float beta_s[C], lg_s[C], g_s[C], tail_s[C];        // beta_i, log g_i, G_i, G_last / G_i
+  const int blocks_e = (a.E + 15) / 16;
+  const int eb = blockIdx.x % blocks_e, head = blockIdx.x / blocks_e;
+  const int s = seq0 + blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int slice = lane & (KS - 1);
+  const int col = wave * 4 + lane / KS;              // the value column inside the workgroup's 16
+  const int e = eb * 16 + col;
+  const bool live = e < a.E;
+  const int kh = head / (a.H / a.G);
+  const int first = a.q_start[s], last = a.q_start[s + 1];
+  if (first >= last) return;
+  float* S_mem = a.state + (((size_t)a.state_slots[s] * a.H + head) * a.E + (live ? e : 0)) * a.Dk + slice * DPL;
+  const bool held = live && slice * DPL < a.Dk;
+  float S[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; i += 4) {
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (held && slice * DPL + i < a.Dk) v = *reinterpret_cast<const f32x4*>(S_mem + i);
+    S[i] = v[0]; S[i + 1] = v[1]; S[i + 2] = v[2]; S[i + 3] = v[3];
+  }
+  const float rate = -expf(a.A_log[head]);
+  const float dt_bias = a.dt_bias[head];
+
+  // a wave stages tokens wave, wave + 4, wave + 8, wave + 12 of a chunk: their raw rows, in registers
+  float rq[4][4], rk[4][4], rv[4], rb[4], ra[4];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) {
+      const int t = t0 + wave + 4 * ii;
+      const bool in = t < last;
+      const float* row = a.qkv + (size_t)(in ? t : first) * a.ld_qkv;
+      const float* qr = row + a.q_col + (size_t)kh * a.D;
+      const float* kr = row + a.k_col + (size_t)kh * a.D;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = lane + 64 * j;
+        const bool ok = in && d < a.D && d < KS * DPL;
+        rq[ii][j] = ok ? qr[d] : 0.f;
+        rk[ii][j] = ok ? kr[d] : 0.f;
+      }
+      const int ev = eb * 16 + (lane & 15);
+      rv[ii] = in && ev < a.E ? row[a.v_col + (size_t)head * a.E + ev] : 0.f;
+      const float* ab = a.ab + (size_t)(in ? t : first) * a.ld_ab;
+      rb[ii] = ab[a.b_col + head];
+      ra[ii] = ab[a.a_col + head];
+    }
+  };
+  auto stage = [&](int t0) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) {
+      const int i = wave + 4 * ii;
+      const bool in = t0 + i < last;
+      float qq = 0.f, kk = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        qq = __fmaf_rn(rq[ii][j], rq[ii][j], qq);
+        kk = __fmaf_rn(rk[ii][j], rk[ii][j], kk);
+      }
+      qq = tw_wave_sum(qq);
+      kk = tw_wave_sum(kk);
+      const float qn = a.q_scale / sqrtf(qq + 1e-6f), kn = 1.f / sqrtf(kk + 1e-6f);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = lane + 64 * j;
+        if (d < KS * DPL) {
+          q_s[i][(d / DPL) * SL + d % DPL] = rq[ii][j] * qn;
+          k_s[i][(d / DPL) * SL + d % DPL] = rk[ii][j] * kn;
+        }
+      }
+      if (lane < 16) v_s[i][lane] = rv[ii];
+      if (lane == 0) {
+        beta_s[i] = in ? 1.f / (1.f + expf(-rb[ii])) : 0.f;
+        lg_s[i] = in ? rate * delta_softplus(ra[ii] + dt_bias) : 0.f;
+      }
+    }
+  };
+
+  fetch(first);
+  for (int t0 = first; t0 < last; t0 += C) {
+    __syncthreads();                                 // the chunk before has been worked on by every wave
+    stage(t0);
+    if (t0 + C < last) fetch(t0 + C);
+    __syncthreads();
+
+    // ---- the products of the chunk's keys and queries with S0: pk[i] = (S0^T k_i)[column], pq of token `slice` ------
+    float pk[C], pq_own = 0.f;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+      const float* kp = &k_s[i][slice * SL];
+      const float* qp = &q_s[i][slice * SL];
+      float d0 = 0.f, d1 = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int j = 0; j < DPL; j += 4) {
+        const f32x4 kq = *reinterpret_cast<const f32x4*>(kp + j);
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(qp + j);
+        d0 = __fmaf_rn(S[j], kq[0], d0);
+        d1 = __fmaf_rn(S[j + 1], kq[1], d1);
+        d0 = __fmaf_rn(S[j + 2], kq[2], d0);
+        d1 = __fmaf_rn(S[j + 3], kq[3], d1);
+        o0 = __fmaf_rn(S[j], qq[0], o0);
+        o1 = __fmaf_rn(S[j + 1], qq[1], o1);
+        o0 = __fmaf_rn(S[j + 2], qq[2], o0);
+        o1 = __fmaf_rn(S[j + 3], qq[3], o1);
+      }
+      pk[i] = delta_group_sum<KS>(d0 + d1);
+      const float pq = delta_group_sum<KS>(o0 + o1);
+      if (slice == i) pq_own = pq;
+    }
+
+    // ---- the pairs: thread 16 i + j forms k_i . k_j and q_i . k_j and the decay between the two tokens ----------------
+    {
+      const int i = threadIdx.x >> 4, j = threadIdx.x & 15;
+      float kk0 = 0.f, kk1 = 0.f, qk0 = 0.f, qk1 = 0.f;
+#pragma unroll 2
+      for (int sl = 0; sl < KS; ++sl)
+#pragma unroll
+        for (int x = 0; x < DPL; x += 4) {
+          const f32x4 ki = *reinterpret_cast<const f32x4*>(&k_s[i][sl * SL + x]);
+          const f32x4 qi = *reinterpret_cast<const f32x4*>(&q_s[i][sl * SL + x]);
+          const f32x4 kj = *reinterpret_cast<const f32x4*>(&k_s[j][sl * SL + x]);
+          kk0 = __fmaf_rn(ki[0], kj[0], kk0);
+          kk1 = __fmaf_rn(ki[1], kj[1], kk1);
+          kk0 = __fmaf_rn(ki[2], kj[2], kk0);
+          kk1 = __fmaf_rn(ki[3], kj[3], kk1);
+          qk0 = __fmaf_rn(qi[0], kj[0], qk0);
+          qk1 = __fmaf_rn(qi[1], kj[1], qk1);
+          qk0 = __fmaf_rn(qi[2], kj[2], qk0);
+          qk1 = __fmaf_rn(qi[3], kj[3], qk1);
+        }
+      float between = 0.f, upto = 0.f;               // log of G_i / G_j (j <= i), and L_i
+#pragma unroll
+      for (int m = 0; m < C; ++m) {
+        const float lg = lg_s[m];
+        if (m > j && m <= i) between += lg;
+        if (m <= i) upto += lg;
+      }
+      const float decay = expf(between);
+      at_s[j][i] = j < i ? beta_s[i] * decay * (kk0 + kk1) : 0.f;
+      qk_s[i][j] = j <= i ? decay * (qk0 + qk1) : 0.f;
+      if (j == 0) g_s[i] = expf(upto);
+      if (i == C - 1) tail_s[j] = decay;
+    }
+    __syncthreads();
+
+    // ---- the triangular system, for this lane's column (the 16 lanes of a column all solve it) ---------------------
+    float u[C];
+#pragma unroll
+    for (int i = 0; i < C; ++i) u[i] = beta_s[i] * (v_s[i][col] - g_s[i] * pk[i]);
+#pragma unroll
+    for (int j = 0; j < C - 1; ++j) {
+      float arow[C];
+#pragma unroll
+      for (int x = 0; x < C; x += 4) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(&at_s[j][x]);
+        arow[x] = v[0]; arow[x + 1] = v[1]; arow[x + 2] = v[2]; arow[x + 3] = v[3];
+      }
+#pragma unroll
+      for (int i = j + 1; i < C; ++i) u[i] = __fmaf_rn(-arow[i], u[j], u[i]);
+    }
+
+    // ---- the read-out of token `slice` ---------------------------------------------------------------------------------
+    {
+      float o = g_s[slice] * pq_own;
+#pragma unroll
+      for (int x = 0; x < C; x += 4) {
+        const f32x4 w = *reinterpret_cast<const f32x4*>(&qk_s[slice][x]);
+        o = __fmaf_rn(w[0], u[x], o);
+        o = __fmaf_rn(w[1], u[x + 1], o);
+        o = __fmaf_rn(w[2], u[x + 2], o);
+        o = __fmaf_rn(w[3], u[x + 3], o);
+      }
+      if (live && t0 + slice < last) a.out[(size_t)(t0 + slice) * a.ld_out + (size_t)head * a.E + e] = o;
+    }
+
+    // ---- the state behind the chunk --------------------------------------------------------------------------------
+    const float G_last = g_s[C - 1];
+#pragma unroll
+    for (int x = 0; x < DPL; ++x) S[x] *= G_last;
+#pragma unroll
+    for (int j = 0; j < C; ++j) {
+      const float w = tail_s[j] * u[j];
+      const float* kp = &k_s[j][slice * SL];
+#pragma unroll
+      for (int x = 0; x < DPL; x += 4) {
+        const f32x4 kq = *reinterpret_cast<const f32x4*>(kp + x);
+        S[x] = __fmaf_rn(kq[0], w, S[x]);
+        S[x + 1] = __fmaf_rn(kq[1], w, S[x + 1]);
+        S[x + 2] = __fmaf_rn(kq[2], w, S[x + 2]);
+        S[x + 3] = __fmaf_rn(kq[3], w, S[x + 3]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < DPL; i += 4)
+    if (held && slice * DPL + i < a.Dk) *reinterpret_cast<f32x4*>(S_mem + i) = f32x4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+}
+
 extern "C" int tw_delta_rule(const float* qkv, long ld_qkv, int q_col, int k_col, int v_col, const float* ab, long ld_ab,
                              int b_col, int a_col, const float* A_log, const float* dt_bias, float* state,
                              const int* q_start, const int* state_slots, float* out, long ld_out, int seq0, int n_seqs,
-                             int H, int G, int D, int E, int Dk, float q_scale, hipStream_t stream) {
+                             int max_q_len, int H, int G, int D, int E, int Dk, float q_scale, hipStream_t stream) {
   TW_REQUIRE(qkv && ab && A_log && dt_bias && state && q_start && state_slots && out);
   TW_REQUIRE(H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && E > 0 && Dk >= D && Dk % 4 == 0 && Dk <= 256);
+  TW_REQUIRE(max_q_len >= 1);
   TW_REQUIRE(seq0 >= 0 && n_seqs >= 0 && ld_out >= (long)H * E && (uintptr_t)state % 16 == 0);
   TW_REQUIRE(q_col >= 0 && k_col >= 0 && v_col >= 0 && b_col >= 0 && a_col >= 0);
   TW_REQUIRE(ld_qkv >= (long)max(q_col, k_col) + (long)G * D && ld_qkv >= (long)v_col + (long)H * E);
@@ -172,7 +395,13 @@ extern "C" int tw_delta_rule(const float* qkv, long ld_qkv, int q_col, int k_col
   if (n_seqs == 0) return 0;
   DeltaArgs a{qkv, ld_qkv, q_col, k_col, v_col, ab, ld_ab, b_col, a_col, A_log, dt_bias, state, q_start, state_slots,
               out, ld_out, H, G, D, E, Dk, q_scale};
-  if (Dk <= 16) {
+  if (max_q_len > TW_DELTA_WALK_MOST) {
+    // some sequence brings many tokens: every sequence of the step goes through the kernel that solves chunks at once
+    const dim3 grid(H * tw_div_up(E, 16), n_seqs);
+    if (Dk <= 64) delta_chunk_kernel<4><<<grid, 256, 0, stream>>>(a, seq0);
+    else if (Dk <= 128) delta_chunk_kernel<8><<<grid, 256, 0, stream>>>(a, seq0);
+    else delta_chunk_kernel<16><<<grid, 256, 0, stream>>>(a, seq0);
+  } else if (Dk <= 16) {
     delta_walk_kernel<4, 4><<<dim3(H * tw_div_up(E, 64), n_seqs), 256, 0, stream>>>(a, seq0);
   } else {
     const dim3 grid(H * tw_div_up(E, 16), n_seqs);

@@ -67,7 +67,7 @@ _SIGNATURES = {
     "tw_swish_limited_mul": (I, [I, P, P, I, I, F, P]),
     "tw_rmsnorm_pair": (I, [I, P, P, P, P, P, I, I, F, P]),
     "tw_scale_values": (I, [P, L, F, P]),
-    "tw_delta_rule": (I, [P, L, I, I, I, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, I, I, F, P]),
+    "tw_delta_rule": (I, [P, L, I, I, I, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, F, P]),
     "tw_head_norm_gate": (I, [I, P, L, P, L, P, P, L, I, I, I, F, P]),
     "tw_moe_route": (I, [I, P, L, P, I, I, I, I, P, P, P]),
     "tw_moe_capacity": (L, [L, I]),

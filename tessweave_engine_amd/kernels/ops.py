@@ -1050,8 +1050,8 @@ def delta_key_extent(dim):
 
 
 def delta_rule(qkv, q_col, k_col, v_col, ab, b_col, a_col, A_log, dt_bias, state, q_start, state_slots, seq0, n_seqs, out,
-               kv_heads, dim, q_scale):
-    """The gated delta rule over sequences seq0 .. seq0 + n_seqs - 1, token by token from and to state float32
+               kv_heads, dim, q_scale, max_q_len=1):
+    """The gated delta rule over sequences seq0 .. seq0 + n_seqs - 1, from and to state float32
     [requests, H, E, Dk] (a column of S is contiguous; Dk = delta_key_extent(dim)):
 
         q~ = unit(q) * q_scale, k~ = unit(k) (unit: x / sqrt(sum x^2 + 1e-6)), beta = sigmoid(b),
@@ -1059,7 +1059,9 @@ def delta_rule(qkv, q_col, k_col, v_col, ab, b_col, a_col, A_log, dt_bias, state
 
     qkv float32 [n, .]: q of key head j at q_col + j * dim, k at k_col + j * dim, v of head h at v_col + h * E;
     ab float32 [n, .]: b of head h at b_col + h, a at a_col + h; value head h reads key head h // (H / kv_heads).
-    out float32 [n, H * E]."""
+    out float32 [n, H * E]. max_q_len: the most tokens a sequence brings (an upper bound will do). Up to a few tokens
+    a sequence the tokens are walked one by one; beyond, chunks of 16 tokens are solved at once (the same sums in another
+    order: a triangular system a chunk in place of a chain of updates)."""
     n, wq, ld_qkv = _rows(qkv, "qkv")
     na, wa, ld_ab = _rows(ab, "ab")
     _need(qkv.dtype == torch.float32 and ab.dtype == torch.float32 and na == n, "the delta rule reads float32 rows")
@@ -1077,7 +1079,7 @@ def delta_rule(qkv, q_col, k_col, v_col, ab, b_col, a_col, A_log, dt_bias, state
     check(library().tw_delta_rule(_dev(qkv), ld_qkv, int(q_col), int(k_col), int(v_col), _dev(ab), ld_ab, int(b_col), int(a_col),
                                   _dev(A_log), _dev(dt_bias), _dev(state), _dev(q_start, torch.int32, "q_start"),
                                   _dev(state_slots, torch.int32, "state_slots"), _dev(out), ldo, int(seq0), int(n_seqs),
-                                  H, G, D, E, Dk, float(q_scale), _stream()), "delta_rule")
+                                  max(1, int(max_q_len)), H, G, D, E, Dk, float(q_scale), _stream()), "delta_rule")
     return out
 
 

@@ -100,7 +100,7 @@ class GatedDeltaRule(Mixer):
         result = ctx.scratch("delta.o", (n, H * E), torch.float32)
         state = ctx.cache.states[run.cache_slot][self.STATE]
         ops.delta_rule(qkv, col["q"], col["k"], col["v"], proj, col["b"], col["a"], self.A_log, self.dt_bias, state,
-                       ctx.q_start, ctx.state_slots, 0, ctx.n_seqs, result, G, D, D ** -0.5)
+                       ctx.q_start, ctx.state_slots, 0, ctx.n_seqs, result, G, D, D ** -0.5, max_q_len=ctx.max_q_len)
         act = ctx.scratch("delta.act", (n, H * E))
         ops.head_norm_gate(result, proj[:, col["g"]:col["g"] + H * E], self.norm_weight, act, H, E, self.eps)
         self.o.forward(ctx, act, x, residual=x if accumulate else None)

@@ -125,11 +125,13 @@ def plain_delta_heads(q, k, v, b, a, A_log, dt_bias, H, G, D, E):
     return torch.stack(out, 1).reshape(T, H * E)
 
 
+@pytest.mark.parametrize("most", [1, 64], ids=["walked", "chunks_solved"])
 @pytest.mark.parametrize("H,G,D,E", [(4, 2, 20, 24), (3, 3, 40, 72), (2, 1, 13, 10), (1, 1, 128, 128), (2, 2, 256, 16), (8, 1, 64, 64)])
-def test_delta_rule_over_cut_sequences_in_reused_slots(device, H, G, D, E):
+def test_delta_rule_over_cut_sequences_in_reused_slots(device, H, G, D, E, most):
     """Three sequences cut differently over four steps (portions of 37 and 21 tokens across chunks of the kernel, two
     tokens, single tokens), the state carried in slots that held another request before. Decays near one: what the
-    first tokens wrote still weighs at the end."""
+    first tokens wrote still weighs at the end. Once with every token walked in turn, once with every step (its single
+    tokens too) through the kernel that solves 16 tokens at once."""
     from tessweave_engine_amd.kernels import ops
     g = torch.Generator().manual_seed(H * 100 + D)
     lens = {"a": 60, "b": 25, "c": 9}
@@ -153,7 +155,8 @@ def test_delta_rule_over_cut_sequences_in_reused_slots(device, H, G, D, E):
         starts = np.cumsum([0] + [n for _, n in parts]).tolist()
         out = torch.full((qkv.shape[0], H * E), float("nan"), device=device)
         ops.delta_rule(qkv, 0, G * D, 2 * G * D, gates, 1, 1 + H, A_log.to(device), dt_bias.to(device), state,
-                       ints(starts, device), ints([slot[k] for k, _ in parts], device), 0, len(parts), out, G, D, D ** -0.5)
+                       ints(starts, device), ints([slot[k] for k, _ in parts], device), 0, len(parts), out, G, D, D ** -0.5,
+                       max_q_len=most)
         for i, (k, n) in enumerate(parts):
             got[k].append(out[starts[i]:starts[i] + n].cpu())
             at[k] += n
@@ -165,7 +168,7 @@ def test_delta_rule_over_cut_sequences_in_reused_slots(device, H, G, D, E):
     state[slot["a"]] = 0
     out = torch.empty(lens["c"], H * E, device=device)
     ops.delta_rule(rows["c"].to(device), 0, G * D, 2 * G * D, ab["c"].to(device), 1, 1 + H, A_log.to(device), dt_bias.to(device), state,
-                   ints([0, lens["c"]], device), ints([slot["a"]], device), 0, 1, out, G, D, D ** -0.5)
+                   ints([0, lens["c"]], device), ints([slot["a"]], device), 0, 1, out, G, D, D ** -0.5, max_q_len=most)
     assert (out.cpu().double() - want["c"]).abs().max() < 2e-5 * max(1.0, want["c"].abs().max().item())
 
 
