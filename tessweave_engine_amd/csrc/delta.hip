@@ -173,6 +173,14 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) 
 // head); thread 16 i + j also forms the pair (i, j) of A and of the read-out's matrix. Tokens behind a sequence's end
 // are staged as zeros with beta = 0 and g = 1: they change nothing. The next chunk's rows are on their way from memory
 // while this one is worked on.
+// The waves of a workgroup meet once each one's LDS traffic is done. (Unlike __syncthreads() this does not wait for loads
+// from memory: the next chunk's rows stay on their way across it.)
+__device__ __forceinline__ void delta_lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 template <int DPL>
 __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0) {
   constexpr int KS = 16, C = 16, SL = DPL + 4;
@@ -254,19 +262,25 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
         }
       }
       if (lane < 16) v_s[i][lane] = rv[ii];
-      if (lane == 0) {
-        beta_s[i] = in ? 1.f / (1.f + expf(-rb[ii])) : 0.f;
-        lg_s[i] = in ? rate * delta_softplus(ra[ii] + dt_bias) : 0.f;
-      }
+    }
+    // the gates of the wave's four tokens, one lane a token (every lane holds all four tokens' b and a)
+    const int mine = lane & 3;
+    const float b = mine == 0 ? rb[0] : mine == 1 ? rb[1] : mine == 2 ? rb[2] : rb[3];
+    const float x = mine == 0 ? ra[0] : mine == 1 ? ra[1] : mine == 2 ? ra[2] : ra[3];
+    if (lane < 4) {
+      const int i = wave + 4 * mine;
+      const bool in = t0 + i < last;
+      beta_s[i] = in ? 1.f / (1.f + expf(-b)) : 0.f;
+      lg_s[i] = in ? rate * delta_softplus(x + dt_bias) : 0.f;
     }
   };
 
   fetch(first);
   for (int t0 = first; t0 < last; t0 += C) {
-    __syncthreads();                                 // the chunk before has been worked on by every wave
+    delta_lds_barrier();                             // the chunk before has been worked on by every wave
     stage(t0);
     if (t0 + C < last) fetch(t0 + C);
-    __syncthreads();
+    delta_lds_barrier();
 
     // ---- the products of the chunk's keys and queries with S0: pk[i] = (S0^T k_i)[column], pq of token `slice` ------
     float pk[C], pq_own = 0.f;
@@ -326,7 +340,7 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
       if (j == 0) g_s[i] = expf(upto);
       if (i == C - 1) tail_s[j] = decay;
     }
-    __syncthreads();
+    delta_lds_barrier();
 
     // ---- the triangular system, for this lane's column (the 16 lanes of a column all solve it) ---------------------
     float u[C];

@@ -662,20 +662,63 @@ extern "C" int tw_swish_limited_mul(int dtype, const void* gu, void* out, int n,
 
 // ---- two RMS norms of the same rows: out1 = unit(x) * w1, out2 = unit(x) * w2 (out2 and w2 may be null) --------------
 // For arrangements whose sublayers all read norms of the same stream: the row is read and its statistic formed once.
-template <typename T>
+__device__ __forceinline__ void pair_store4(float* dst, const float (&v)[4]) {
+  *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+}
+__device__ __forceinline__ void pair_store4(bf16_t* dst, const float (&v)[4]) {
+  *reinterpret_cast<bf16x4*>(dst) = bf16x4{(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+}
+
+// VEC: rows of a multiple of 4 and at most 4,096 elements at 16-byte aligned addresses: a thread keeps its (up to four)
+// groups of four elements in registers, so the row is read once and every load is on its way before the first is used.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_pair_kernel(const float* __restrict__ x, const float* __restrict__ w1,
                                                            const float* __restrict__ w2, T* __restrict__ out1,
                                                            T* __restrict__ out2, int hidden, float eps) {
   __shared__ float red[16];
   const float* row = x + (size_t)blockIdx.x * hidden;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) ss = __fmaf_rn(row[c], row[c], ss);
-  ss = tw_block_sum(ss, red);
-  const float rinv = 1.f / sqrtf(ss / (float)hidden + eps);
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-    const float u = row[c] * rinv;
-    out1[(size_t)blockIdx.x * hidden + c] = tw_from_float<T>(u * w1[c]);
-    if (out2) out2[(size_t)blockIdx.x * hidden + c] = tw_from_float<T>(u * w2[c]);
+  if constexpr (VEC) {
+    f32x4 v[4], a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = (threadIdx.x + 256 * i) * 4;
+      v[i] = a[i] = b[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (c < hidden) {
+        v[i] = *reinterpret_cast<const f32x4*>(row + c);
+        a[i] = *reinterpret_cast<const f32x4*>(w1 + c);
+        if (w2) b[i] = *reinterpret_cast<const f32x4*>(w2 + c);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ss = __fmaf_rn(v[i][j], v[i][j], ss);
+    ss = tw_block_sum(ss, red);
+    const float rinv = 1.f / sqrtf(ss / (float)hidden + eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = (threadIdx.x + 256 * i) * 4;
+      if (c >= hidden) continue;
+      float o1[4], o2[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float u = v[i][j] * rinv;
+        o1[j] = u * a[i][j];
+        o2[j] = u * b[i][j];
+      }
+      pair_store4(out1 + (size_t)blockIdx.x * hidden + c, o1);
+      if (out2) pair_store4(out2 + (size_t)blockIdx.x * hidden + c, o2);
+    }
+  } else {
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) ss = __fmaf_rn(row[c], row[c], ss);
+    ss = tw_block_sum(ss, red);
+    const float rinv = 1.f / sqrtf(ss / (float)hidden + eps);
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+      const float u = row[c] * rinv;
+      out1[(size_t)blockIdx.x * hidden + c] = tw_from_float<T>(u * w1[c]);
+      if (out2) out2[(size_t)blockIdx.x * hidden + c] = tw_from_float<T>(u * w2[c]);
+    }
   }
 }
 
@@ -683,12 +726,17 @@ extern "C" int tw_rmsnorm_pair(int dtype, const float* x, const float* w1, const
                                int hidden, float eps, hipStream_t stream) {
   TW_REQUIRE(x && w1 && out1 && ((w2 != nullptr) == (out2 != nullptr)) && n >= 0 && hidden > 0 && eps > 0.f);
   if (n == 0) return 0;
-  if (dtype == TW_DTYPE_F32)
-    rmsnorm_pair_kernel<float><<<n, 256, 0, stream>>>(x, w1, w2, (float*)out1, (float*)out2, hidden, eps);
-  else if (dtype == TW_DTYPE_BF16)
-    rmsnorm_pair_kernel<bf16_t><<<n, 256, 0, stream>>>(x, w1, w2, (bf16_t*)out1, (bf16_t*)out2, hidden, eps);
-  else
+  const bool vec = hidden % 4 == 0 && hidden <= 4096 && (uintptr_t)x % 16 == 0 && (uintptr_t)w1 % 16 == 0 &&
+                   (uintptr_t)w2 % 16 == 0 && (uintptr_t)out1 % 16 == 0 && (uintptr_t)out2 % 16 == 0;
+  if (dtype == TW_DTYPE_F32) {
+    if (vec) rmsnorm_pair_kernel<float, true><<<n, 256, 0, stream>>>(x, w1, w2, (float*)out1, (float*)out2, hidden, eps);
+    else rmsnorm_pair_kernel<float, false><<<n, 256, 0, stream>>>(x, w1, w2, (float*)out1, (float*)out2, hidden, eps);
+  } else if (dtype == TW_DTYPE_BF16) {
+    if (vec) rmsnorm_pair_kernel<bf16_t, true><<<n, 256, 0, stream>>>(x, w1, w2, (bf16_t*)out1, (bf16_t*)out2, hidden, eps);
+    else rmsnorm_pair_kernel<bf16_t, false><<<n, 256, 0, stream>>>(x, w1, w2, (bf16_t*)out1, (bf16_t*)out2, hidden, eps);
+  } else {
     return TW_ERR_BAD_ARGUMENT;
+  }
   return TW_LAUNCH_RESULT();
 }
 

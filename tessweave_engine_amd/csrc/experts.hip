@@ -276,13 +276,24 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
 }
 
 // ---- combine: x[token] += its experts' rows, in the order of its choices ------------------------------------------
+// A workgroup takes 1,024 columns of a row, four a thread where rows and addresses allow 16-byte accesses.
+template <bool VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long ld_x, const float* __restrict__ ys,
                                                           long ld_y, const int* __restrict__ pos, int C, int top) {
   const int row = blockIdx.x;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float sum = 0.f;
-    for (int r = 0; r < top; ++r) sum += ys[(size_t)pos[(size_t)row * top + r] * ld_y + c];
-    x[(size_t)row * ld_x + c] += sum;
+  const int c = blockIdx.y * 1024 + threadIdx.x * 4;
+  if (c >= C) return;
+  if constexpr (VEC) {
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < top; ++r) sum += *reinterpret_cast<const f32x4*>(ys + (size_t)pos[(size_t)row * top + r] * ld_y + c);
+    f32x4* dst = reinterpret_cast<f32x4*>(x + (size_t)row * ld_x + c);
+    *dst += sum;
+  } else {
+    for (int j = 0; j < 4 && c + j < C; ++j) {
+      float sum = 0.f;
+      for (int r = 0; r < top; ++r) sum += ys[(size_t)pos[(size_t)row * top + r] * ld_y + c + j];
+      x[(size_t)row * ld_x + c + j] += sum;
+    }
   }
 }
 
@@ -349,6 +360,10 @@ extern "C" int tw_moe_experts(int dtype, const void* h, long ld_h, const int* id
   } else {
     return TW_ERR_BAD_ARGUMENT;
   }
-  moe_combine_kernel<<<n, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top);
+  const dim3 combine_grid(n, tw_div_up(C, 1024));
+  if (C % 4 == 0 && ld_x % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)ys % 16 == 0)
+    moe_combine_kernel<true><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top);
+  else
+    moe_combine_kernel<false><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top);
   return TW_LAUNCH_RESULT();
 }
