@@ -160,19 +160,6 @@ __global__ __launch_bounds__(256) void delta_walk_kernel(DeltaArgs a, int seq0) 
     if (held && slice * DPL + i < a.Dk) *reinterpret_cast<f32x4*>(S_mem + i) = f32x4{S[i], S[i + 1], S[i + 2], S[i + 3]};
 }
 
-// ---- many tokens a sequence: chunks of 16 tokens, each solved at once ----------------------------------------------
-// Inside a chunk with state S0 at its start, L_i = sum_{m <= i} log g_m (so that G_i = exp(L_i) and every quotient
-// G_i / G_j, j <= i, is an exponential of a sum of logarithms that are at most 0):
-//   u_i = beta_i (v_i - G_i S0^T k_i) - sum_{j < i} A_ij u_j,      A_ij = beta_i (G_i / G_j) (k_i . k_j)
-//   o_i = G_i S0^T q_i + sum_{j <= i} (G_i / G_j) (q_i . k_j) u_j
-//   S   = G_last S0 + sum_j (G_last / G_j) k_j u_j^T
-// which is the token-by-token rule written out. The products with S0 of all 16 tokens are independent of each other
-// (the walk's are a chain), the triangular system is solved by substitution per value column (after u_j is final every
-// later row takes its term off: one multiply-add deep a token), and the state is read and written once a chunk.
-// Lanes as in the walk with 16 slices: lane = 16 * column + slice; a workgroup owns 16 value columns of one (sequence,
-// head); thread 16 i + j also forms the pair (i, j) of A and of the read-out's matrix. Tokens behind a sequence's end
-// are staged as zeros with beta = 0 and g = 1: they change nothing. The next chunk's rows are on their way from memory
-// while this one is worked on.
 // The waves of a workgroup meet once each one's LDS traffic is done. (Unlike __syncthreads() this does not wait for loads
 // from memory: the next chunk's rows stay on their way across it.)
 __device__ __forceinline__ void delta_lds_barrier() {
@@ -181,14 +168,33 @@ __device__ __forceinline__ void delta_lds_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <int DPL>
+// ---- many tokens a sequence: chunks of 16 tokens, each solved at once ----------------------------------------------
+// Inside a chunk with state S0 at its start, L_i = sum_{m <= i} log g_m (so that G_i = exp(L_i) and every quotient
+// G_i / G_j, j <= i, is an exponential of a sum of logarithms that are at most 0):
+//   u_i = beta_i (v_i - G_i S0^T k_i) - sum_{j < i} A_ij u_j,      A_ij = beta_i (G_i / G_j) (k_i . k_j)
+//   o_i = G_i S0^T q_i + sum_{j <= i} (G_i / G_j) (q_i . k_j) u_j
+//   S   = G_last S0 + sum_j (G_last / G_j) k_j u_j^T
+// which is the token-by-token rule written out. All products are float32 on the matrix unit (16x16x4). A workgroup
+// owns 16 value columns of one (sequence, head); its four waves own a quarter of the key elements each (NT tiles of 16),
+// and a wave's part of S stays in registers in the layout that is both the B operand of K S and the accumulator of
+// K^T W: lane (c, g) holds S[16 tile + 4 g + j][c]. Per chunk: the waves form their parts of K S0, Q S0, K K^T and
+// Q K^T from the same fragments (the key rows of a chunk are the A operand of the first and both operands of the third),
+// the parts meet in LDS and thread 16 i + j adds them up for the pair (i, j) and puts decay and beta on; every lane solves
+// the triangular system of its column by substitution (after u_j is final every later row takes its term off: one
+// multiply-add deep a token); one wave reads the chunk's outputs out (one more product), every wave updates its part
+// of S. Tokens behind a sequence's end are staged as zeros with beta = 0 and g = 1: they change nothing. The next
+// chunk's rows are on their way from memory while this one is worked on.
+template <int NT>
 __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0) {
-  constexpr int KS = 16, C = 16, SL = DPL + 4;
-  constexpr int ROW = KS * SL + 4;                   // (+ 4: the 16 rows a read of the pair products meets lie in different banks)
+  constexpr int C = 16, DP = 64 * NT;                // key elements, rounded up: 16 NT a wave
+  constexpr int ROW = DP + 4;                        // (+ 4: the four token rows a transposed read meets lie 16 banks apart)
   constexpr int PW = C + 4;
   __shared__ __attribute__((aligned(16))) float q_s[C][ROW];
   __shared__ __attribute__((aligned(16))) float k_s[C][ROW];
-  __shared__ __attribute__((aligned(16))) float v_s[C][16];
+  __shared__ __attribute__((aligned(16))) float part_s[4][4][C][C];   // [wave][K S0, Q S0, K K^T, Q K^T][row][column]
+  __shared__ __attribute__((aligned(16))) float v_s[C][C];
+  __shared__ __attribute__((aligned(16))) float pk_s[C][C];      // (S0^T k_i)[column]
+  __shared__ __attribute__((aligned(16))) float pq_s[C][C];
   __shared__ __attribute__((aligned(16))) float at_s[C][PW];     // at_s[j][i] = A_ij (0 unless j < i)
   __shared__ __attribute__((aligned(16))) float qk_s[C][PW];     // qk_s[i][j] = (G_i / G_j) (q_i . k_j) (0 unless j <= i)
   __shared__ float beta_s[C], lg_s[C], g_s[C], tail_s[C];        // beta_i, log g_i, G_i, G_last / G_i
@@ -196,27 +202,26 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
   const int eb = blockIdx.x % blocks_e, head = blockIdx.x / blocks_e;
   const int s = seq0 + blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int slice = lane & (KS - 1);
-  const int col = wave * 4 + lane / KS;              // the value column inside the workgroup's 16
-  const int e = eb * 16 + col;
+  const int r = lane & 15, g = lane >> 4;
+  const int e = eb * 16 + r;                         // this lane's value column
   const bool live = e < a.E;
   const int kh = head / (a.H / a.G);
   const int first = a.q_start[s], last = a.q_start[s + 1];
   if (first >= last) return;
-  float* S_mem = a.state + (((size_t)a.state_slots[s] * a.H + head) * a.E + (live ? e : 0)) * a.Dk + slice * DPL;
-  const bool held = live && slice * DPL < a.Dk;
-  float S[DPL];
+  const int d_wave = 16 * NT * wave;                 // the wave's first key element
+  float* S_mem = a.state + (((size_t)a.state_slots[s] * a.H + head) * a.E + (live ? e : 0)) * a.Dk;
+  f32x4 S[NT];
 #pragma unroll
-  for (int i = 0; i < DPL; i += 4) {
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (held && slice * DPL + i < a.Dk) v = *reinterpret_cast<const f32x4*>(S_mem + i);
-    S[i] = v[0]; S[i + 1] = v[1]; S[i + 2] = v[2]; S[i + 3] = v[3];
+  for (int mm = 0; mm < NT; ++mm) {
+    const int d0 = d_wave + 16 * mm + 4 * g;
+    S[mm] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (live && d0 < a.Dk) S[mm] = *reinterpret_cast<const f32x4*>(S_mem + d0);
   }
   const float rate = -expf(a.A_log[head]);
   const float dt_bias = a.dt_bias[head];
 
   // a wave stages tokens wave, wave + 4, wave + 8, wave + 12 of a chunk: their raw rows, in registers
-  float rq[4][4], rk[4][4], rv[4], rb[4], ra[4];
+  float rq[4][NT], rk[4][NT], rv[4], rb[4], ra[4];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii) {
@@ -226,13 +231,13 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
       const float* qr = row + a.q_col + (size_t)kh * a.D;
       const float* kr = row + a.k_col + (size_t)kh * a.D;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NT; ++j) {
         const int d = lane + 64 * j;
-        const bool ok = in && d < a.D && d < KS * DPL;
+        const bool ok = in && d < a.D;
         rq[ii][j] = ok ? qr[d] : 0.f;
         rk[ii][j] = ok ? kr[d] : 0.f;
       }
-      const int ev = eb * 16 + (lane & 15);
+      const int ev = eb * 16 + r;
       rv[ii] = in && ev < a.E ? row[a.v_col + (size_t)head * a.E + ev] : 0.f;
       const float* ab = a.ab + (size_t)(in ? t : first) * a.ld_ab;
       rb[ii] = ab[a.b_col + head];
@@ -243,10 +248,9 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii) {
       const int i = wave + 4 * ii;
-      const bool in = t0 + i < last;
       float qq = 0.f, kk = 0.f;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NT; ++j) {
         qq = __fmaf_rn(rq[ii][j], rq[ii][j], qq);
         kk = __fmaf_rn(rk[ii][j], rk[ii][j], kk);
       }
@@ -254,12 +258,9 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
       kk = tw_wave_sum(kk);
       const float qn = a.q_scale / sqrtf(qq + 1e-6f), kn = 1.f / sqrtf(kk + 1e-6f);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int d = lane + 64 * j;
-        if (d < KS * DPL) {
-          q_s[i][(d / DPL) * SL + d % DPL] = rq[ii][j] * qn;
-          k_s[i][(d / DPL) * SL + d % DPL] = rk[ii][j] * kn;
-        }
+      for (int j = 0; j < NT; ++j) {
+        q_s[i][lane + 64 * j] = rq[ii][j] * qn;
+        k_s[i][lane + 64 * j] = rk[ii][j] * kn;
       }
       if (lane < 16) v_s[i][lane] = rv[ii];
     }
@@ -282,51 +283,34 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
     if (t0 + C < last) fetch(t0 + C);
     delta_lds_barrier();
 
-    // ---- the products of the chunk's keys and queries with S0: pk[i] = (S0^T k_i)[column], pq of token `slice` ------
-    float pk[C], pq_own = 0.f;
+    // ---- this wave's parts of the four products -----------------------------------------------------------------------
+    {
+      f32x4 pk = {0.f, 0.f, 0.f, 0.f}, pq = pk, kk = pk, qk = pk;
 #pragma unroll
-    for (int i = 0; i < C; ++i) {
-      const float* kp = &k_s[i][slice * SL];
-      const float* qp = &q_s[i][slice * SL];
-      float d0 = 0.f, d1 = 0.f, o0 = 0.f, o1 = 0.f;
-#pragma unroll
-      for (int j = 0; j < DPL; j += 4) {
-        const f32x4 kq = *reinterpret_cast<const f32x4*>(kp + j);
-        const f32x4 qq = *reinterpret_cast<const f32x4*>(qp + j);
-        d0 = __fmaf_rn(S[j], kq[0], d0);
-        d1 = __fmaf_rn(S[j + 1], kq[1], d1);
-        d0 = __fmaf_rn(S[j + 2], kq[2], d0);
-        d1 = __fmaf_rn(S[j + 3], kq[3], d1);
-        o0 = __fmaf_rn(S[j], qq[0], o0);
-        o1 = __fmaf_rn(S[j + 1], qq[1], o1);
-        o0 = __fmaf_rn(S[j + 2], qq[2], o0);
-        o1 = __fmaf_rn(S[j + 3], qq[3], o1);
+      for (int mm = 0; mm < NT; ++mm) {
+        const f32x4 kf = *reinterpret_cast<const f32x4*>(&k_s[r][d_wave + 16 * mm + 4 * g]);
+        const f32x4 qf = *reinterpret_cast<const f32x4*>(&q_s[r][d_wave + 16 * mm + 4 * g]);
+        tw_mma16(pk, kf, S[mm]);                     // [token][column]
+        tw_mma16(pq, qf, S[mm]);
+        tw_mma16(kk, kf, kf);                        // [token i][token j]
+        tw_mma16(qk, qf, kf);
       }
-      pk[i] = delta_group_sum<KS>(d0 + d1);
-      const float pq = delta_group_sum<KS>(o0 + o1);
-      if (slice == i) pq_own = pq;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        part_s[wave][0][4 * g + j][r] = pk[j];
+        part_s[wave][1][4 * g + j][r] = pq[j];
+        part_s[wave][2][4 * g + j][r] = kk[j];
+        part_s[wave][3][4 * g + j][r] = qk[j];
+      }
     }
+    delta_lds_barrier();
 
-    // ---- the pairs: thread 16 i + j forms k_i . k_j and q_i . k_j and the decay between the two tokens ----------------
+    // ---- thread 16 i + j adds the waves' parts up (in their order) and puts the decay between tokens i and j on -----
     {
       const int i = threadIdx.x >> 4, j = threadIdx.x & 15;
-      float kk0 = 0.f, kk1 = 0.f, qk0 = 0.f, qk1 = 0.f;
-#pragma unroll 2
-      for (int sl = 0; sl < KS; ++sl)
+      float sum[4];
 #pragma unroll
-        for (int x = 0; x < DPL; x += 4) {
-          const f32x4 ki = *reinterpret_cast<const f32x4*>(&k_s[i][sl * SL + x]);
-          const f32x4 qi = *reinterpret_cast<const f32x4*>(&q_s[i][sl * SL + x]);
-          const f32x4 kj = *reinterpret_cast<const f32x4*>(&k_s[j][sl * SL + x]);
-          kk0 = __fmaf_rn(ki[0], kj[0], kk0);
-          kk1 = __fmaf_rn(ki[1], kj[1], kk1);
-          kk0 = __fmaf_rn(ki[2], kj[2], kk0);
-          kk1 = __fmaf_rn(ki[3], kj[3], kk1);
-          qk0 = __fmaf_rn(qi[0], kj[0], qk0);
-          qk1 = __fmaf_rn(qi[1], kj[1], qk1);
-          qk0 = __fmaf_rn(qi[2], kj[2], qk0);
-          qk1 = __fmaf_rn(qi[3], kj[3], qk1);
-        }
+      for (int t = 0; t < 4; ++t) sum[t] = (part_s[0][t][i][j] + part_s[1][t][i][j]) + (part_s[2][t][i][j] + part_s[3][t][i][j]);
       float between = 0.f, upto = 0.f;               // log of G_i / G_j (j <= i), and L_i
 #pragma unroll
       for (int m = 0; m < C; ++m) {
@@ -335,17 +319,19 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
         if (m <= i) upto += lg;
       }
       const float decay = expf(between);
-      at_s[j][i] = j < i ? beta_s[i] * decay * (kk0 + kk1) : 0.f;
-      qk_s[i][j] = j <= i ? decay * (qk0 + qk1) : 0.f;
+      pk_s[i][j] = sum[0];
+      pq_s[i][j] = sum[1];
+      at_s[j][i] = j < i ? beta_s[i] * decay * sum[2] : 0.f;
+      qk_s[i][j] = j <= i ? decay * sum[3] : 0.f;
       if (j == 0) g_s[i] = expf(upto);
       if (i == C - 1) tail_s[j] = decay;
     }
     delta_lds_barrier();
 
-    // ---- the triangular system, for this lane's column (the 16 lanes of a column all solve it) ---------------------
+    // ---- the triangular system of this lane's column (the lanes of a column, in every wave, all solve it) -----------
     float u[C];
 #pragma unroll
-    for (int i = 0; i < C; ++i) u[i] = beta_s[i] * (v_s[i][col] - g_s[i] * pk[i]);
+    for (int i = 0; i < C; ++i) u[i] = beta_s[i] * (v_s[i][r] - g_s[i] * pk_s[i][r]);
 #pragma unroll
     for (int j = 0; j < C - 1; ++j) {
       float arow[C];
@@ -357,42 +343,44 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
 #pragma unroll
       for (int i = j + 1; i < C; ++i) u[i] = __fmaf_rn(-arow[i], u[j], u[i]);
     }
-
-    // ---- the read-out of token `slice` ---------------------------------------------------------------------------------
-    {
-      float o = g_s[slice] * pq_own;
+    // u of tokens 4 g .. 4 g + 3: the B operand of the two products over tokens
+    f32x4 ub;
 #pragma unroll
-      for (int x = 0; x < C; x += 4) {
-        const f32x4 w = *reinterpret_cast<const f32x4*>(&qk_s[slice][x]);
-        o = __fmaf_rn(w[0], u[x], o);
-        o = __fmaf_rn(w[1], u[x + 1], o);
-        o = __fmaf_rn(w[2], u[x + 2], o);
-        o = __fmaf_rn(w[3], u[x + 3], o);
+    for (int j = 0; j < 4; ++j) ub[j] = g == 0 ? u[j] : g == 1 ? u[4 + j] : g == 2 ? u[8 + j] : u[12 + j];
+
+    // ---- the read-out: o_i = G_i (S0^T q_i) + sum_j qk[i][j] u_j, by the chunk's wave in turn -------------------------
+    if (wave == ((t0 - first) / C & 3)) {
+      f32x4 o = {0.f, 0.f, 0.f, 0.f};
+      const f32x4 w = *reinterpret_cast<const f32x4*>(&qk_s[r][4 * g]);
+      tw_mma16(o, w, ub);                            // [token i][column]
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        const float out = __fmaf_rn(g_s[i], pq_s[i][r], o[j]);
+        if (live && t0 + i < last) a.out[(size_t)(t0 + i) * a.ld_out + (size_t)head * a.E + e] = out;
       }
-      if (live && t0 + slice < last) a.out[(size_t)(t0 + slice) * a.ld_out + (size_t)head * a.E + e] = o;
     }
 
-    // ---- the state behind the chunk --------------------------------------------------------------------------------
+    // ---- the state behind the chunk: S <- G_last S + K^T diag(G_last / G_j) U ----------------------------------------
     const float G_last = g_s[C - 1];
+    f32x4 wb;
 #pragma unroll
-    for (int x = 0; x < DPL; ++x) S[x] *= G_last;
+    for (int j = 0; j < 4; ++j) wb[j] = tail_s[4 * g + j] * ub[j];
 #pragma unroll
-    for (int j = 0; j < C; ++j) {
-      const float w = tail_s[j] * u[j];
-      const float* kp = &k_s[j][slice * SL];
+    for (int mm = 0; mm < NT; ++mm) {
+      f32x4 kt;                                      // A operand: row = key element 16 tile + r, reduction = token 4 g + j
 #pragma unroll
-      for (int x = 0; x < DPL; x += 4) {
-        const f32x4 kq = *reinterpret_cast<const f32x4*>(kp + x);
-        S[x] = __fmaf_rn(kq[0], w, S[x]);
-        S[x + 1] = __fmaf_rn(kq[1], w, S[x + 1]);
-        S[x + 2] = __fmaf_rn(kq[2], w, S[x + 2]);
-        S[x + 3] = __fmaf_rn(kq[3], w, S[x + 3]);
-      }
+      for (int j = 0; j < 4; ++j) kt[j] = k_s[4 * g + j][d_wave + 16 * mm + r];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) S[mm][j] *= G_last;
+      tw_mma16(S[mm], kt, wb);
     }
   }
 #pragma unroll
-  for (int i = 0; i < DPL; i += 4)
-    if (held && slice * DPL + i < a.Dk) *reinterpret_cast<f32x4*>(S_mem + i) = f32x4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+  for (int mm = 0; mm < NT; ++mm) {
+    const int d0 = d_wave + 16 * mm + 4 * g;
+    if (live && d0 < a.Dk) *reinterpret_cast<f32x4*>(S_mem + d0) = S[mm];
+  }
 }
 
 extern "C" int tw_delta_rule(const float* qkv, long ld_qkv, int q_col, int k_col, int v_col, const float* ab, long ld_ab,
@@ -412,9 +400,9 @@ extern "C" int tw_delta_rule(const float* qkv, long ld_qkv, int q_col, int k_col
   if (max_q_len > TW_DELTA_WALK_MOST) {
     // some sequence brings many tokens: every sequence of the step goes through the kernel that solves chunks at once
     const dim3 grid(H * tw_div_up(E, 16), n_seqs);
-    if (Dk <= 64) delta_chunk_kernel<4><<<grid, 256, 0, stream>>>(a, seq0);
-    else if (Dk <= 128) delta_chunk_kernel<8><<<grid, 256, 0, stream>>>(a, seq0);
-    else delta_chunk_kernel<16><<<grid, 256, 0, stream>>>(a, seq0);
+    if (Dk <= 64) delta_chunk_kernel<1><<<grid, 256, 0, stream>>>(a, seq0);
+    else if (Dk <= 128) delta_chunk_kernel<2><<<grid, 256, 0, stream>>>(a, seq0);
+    else delta_chunk_kernel<4><<<grid, 256, 0, stream>>>(a, seq0);
   } else if (Dk <= 16) {
     delta_walk_kernel<4, 4><<<dim3(H * tw_div_up(E, 64), n_seqs), 256, 0, stream>>>(a, seq0);
   } else {
