@@ -179,7 +179,8 @@ __device__ __forceinline__ void delta_lds_barrier() {
 // and a wave's part of S stays in registers in the layout that is both the B operand of K S and the accumulator of
 // K^T W: lane (c, g) holds S[16 tile + 4 g + j][c]. Per chunk: the waves form their parts of K S0, Q S0, K K^T and
 // Q K^T from the same fragments (the key rows of a chunk are the A operand of the first and both operands of the third),
-// the parts meet in LDS and thread 16 i + j adds them up for the pair (i, j) and puts decay and beta on; every lane solves
+// the parts meet in LDS and thread 16 i + j adds them up for the pair (i, j) and puts decay, beta and the unit norms on
+// (q and k are multiplied as they come; their squared lengths are the diagonals of K K^T and of one more product, Q Q^T); every lane solves
 // the triangular system of its column by substitution (after u_j is final every later row takes its term off: one
 // multiply-add deep a token); one wave reads the chunk's outputs out (one more product), every wave updates its part
 // of S. Tokens behind a sequence's end are staged as zeros with beta = 0 and g = 1: they change nothing. The next
@@ -191,13 +192,13 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
   constexpr int PW = C + 4;
   __shared__ __attribute__((aligned(16))) float q_s[C][ROW];
   __shared__ __attribute__((aligned(16))) float k_s[C][ROW];
-  __shared__ __attribute__((aligned(16))) float part_s[4][4][C][C];   // [wave][K S0, Q S0, K K^T, Q K^T][row][column]
+  __shared__ __attribute__((aligned(16))) float part_s[4][5][C][C];   // [wave][K S0, Q S0, K K^T, Q K^T, Q Q^T][row][column]
   __shared__ __attribute__((aligned(16))) float v_s[C][C];
   __shared__ __attribute__((aligned(16))) float pk_s[C][C];      // (S0^T k_i)[column]
   __shared__ __attribute__((aligned(16))) float pq_s[C][C];
   __shared__ __attribute__((aligned(16))) float at_s[C][PW];     // at_s[j][i] = A_ij (0 unless j < i)
   __shared__ __attribute__((aligned(16))) float qk_s[C][PW];     // qk_s[i][j] = (G_i / G_j) (q_i . k_j) (0 unless j <= i)
-  __shared__ float beta_s[C], lg_s[C], g_s[C], tail_s[C];        // beta_i, log g_i, G_i, G_last / G_i
+  __shared__ float beta_s[C], lg_s[C], g_s[C], tail_s[C];        // beta_i, log g_i, G_i, G_last / G_i * (1 / |k_i|)
   const int blocks_e = (a.E + 15) / 16;
   const int eb = blockIdx.x % blocks_e, head = blockIdx.x / blocks_e;
   const int s = seq0 + blockIdx.y;
@@ -248,19 +249,10 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii) {
       const int i = wave + 4 * ii;
-      float qq = 0.f, kk = 0.f;
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        qq = __fmaf_rn(rq[ii][j], rq[ii][j], qq);
-        kk = __fmaf_rn(rk[ii][j], rk[ii][j], kk);
-      }
-      qq = tw_wave_sum(qq);
-      kk = tw_wave_sum(kk);
-      const float qn = a.q_scale / sqrtf(qq + 1e-6f), kn = 1.f / sqrtf(kk + 1e-6f);
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        q_s[i][lane + 64 * j] = rq[ii][j] * qn;
-        k_s[i][lane + 64 * j] = rk[ii][j] * kn;
+        q_s[i][lane + 64 * j] = rq[ii][j];           // (as they come: the unit norms are put on the products)
+        k_s[i][lane + 64 * j] = rk[ii][j];
       }
       if (lane < 16) v_s[i][lane] = rv[ii];
     }
@@ -285,7 +277,7 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
 
     // ---- this wave's parts of the four products -----------------------------------------------------------------------
     {
-      f32x4 pk = {0.f, 0.f, 0.f, 0.f}, pq = pk, kk = pk, qk = pk;
+      f32x4 pk = {0.f, 0.f, 0.f, 0.f}, pq = pk, kk = pk, qk = pk, qq = pk;
 #pragma unroll
       for (int mm = 0; mm < NT; ++mm) {
         const f32x4 kf = *reinterpret_cast<const f32x4*>(&k_s[r][d_wave + 16 * mm + 4 * g]);
@@ -294,6 +286,7 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
         tw_mma16(pq, qf, S[mm]);
         tw_mma16(kk, kf, kf);                        // [token i][token j]
         tw_mma16(qk, qf, kf);
+        tw_mma16(qq, qf, qf);                        // (its diagonal: the queries' squared lengths, as K K^T's are the keys')
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -301,6 +294,7 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
         part_s[wave][1][4 * g + j][r] = pq[j];
         part_s[wave][2][4 * g + j][r] = kk[j];
         part_s[wave][3][4 * g + j][r] = qk[j];
+        part_s[wave][4][4 * g + j][r] = qq[j];
       }
     }
     delta_lds_barrier();
@@ -308,9 +302,15 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
     // ---- thread 16 i + j adds the waves' parts up (in their order) and puts the decay between tokens i and j on -----
     {
       const int i = threadIdx.x >> 4, j = threadIdx.x & 15;
+      auto whole = [&](int t, int row, int column) {
+        return (part_s[0][t][row][column] + part_s[1][t][row][column]) + (part_s[2][t][row][column] + part_s[3][t][row][column]);
+      };
       float sum[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) sum[t] = (part_s[0][t][i][j] + part_s[1][t][i][j]) + (part_s[2][t][i][j] + part_s[3][t][i][j]);
+      for (int t = 0; t < 4; ++t) sum[t] = whole(t, i, j);
+      // q and k were multiplied as they came: 1 / |k_i|, 1 / |k_j| and q_scale / |q_i| from the diagonals
+      const float kn_i = 1.f / sqrtf(whole(2, i, i) + 1e-6f), kn_j = 1.f / sqrtf(whole(2, j, j) + 1e-6f);
+      const float qn_i = a.q_scale / sqrtf(whole(4, i, i) + 1e-6f);
       float between = 0.f, upto = 0.f;               // log of G_i / G_j (j <= i), and L_i
 #pragma unroll
       for (int m = 0; m < C; ++m) {
@@ -319,12 +319,12 @@ __global__ __launch_bounds__(256) void delta_chunk_kernel(DeltaArgs a, int seq0)
         if (m <= i) upto += lg;
       }
       const float decay = expf(between);
-      pk_s[i][j] = sum[0];
-      pq_s[i][j] = sum[1];
-      at_s[j][i] = j < i ? beta_s[i] * decay * sum[2] : 0.f;
-      qk_s[i][j] = j <= i ? decay * sum[3] : 0.f;
+      pk_s[i][j] = kn_i * sum[0];
+      pq_s[i][j] = qn_i * sum[1];
+      at_s[j][i] = j < i ? beta_s[i] * decay * (kn_i * kn_j) * sum[2] : 0.f;
+      qk_s[i][j] = j <= i ? decay * (qn_i * kn_j) * sum[3] : 0.f;
       if (j == 0) g_s[i] = expf(upto);
-      if (i == C - 1) tail_s[j] = decay;
+      if (i == C - 1) tail_s[j] = decay * kn_j;
     }
     delta_lds_barrier();
 
