@@ -704,12 +704,15 @@ def test_attn_prefill_random_shapes_with_long_key_ranges(ops, device):
                                                  f"q {qlens} window {window} split {split}: {m}")
 
 
+@pytest.mark.parametrize("d,page,n,q_len", [(32, 8, 75, 9), (128, 16, 700, 260), (256, 16, 330, 70), (80, 8, 300, 150), (64, 4, 90, 20)])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_attn_soft_capped_scores(ops, device, dtype):
+def test_attn_soft_capped_scores(ops, device, dtype, d, page, n, q_len):
     """softcap * tanh(score / softcap) before the softmax, decode and prompt portions, against the formula in
     torch. Queries are long enough that uncapped scores reach several times the cap: without the cap, or with
-    the cap before the scale, the result is wrong by O(1)."""
-    heads, kv_heads, d, page, n, q_len, cap = 4, 2, 32, 8, 75, 9, 5.0
+    the cap before the scale, the result is wrong by O(1). Head sizes and lengths that reach every form of the
+    bfloat16 kernels' loops (whole and partial head sizes, blocks every row sees, blocks at the diagonal and at the
+    sequence's end) and, with pages of four keys, the kernels for every page size."""
+    heads, kv_heads, cap = 4, 2, 5.0
     gen = torch.Generator().manual_seed(8)
     k = torch.randn(n, kv_heads, d, generator=gen).to(dtype).float()
     v = torch.randn(n, kv_heads, d, generator=gen).to(dtype).float()

@@ -61,7 +61,7 @@ def double(weights):
 # ---------------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n,C", [(5, 88), (70, 1000), (3, 4097)])
+@pytest.mark.parametrize("n,C", [(5, 88), (70, 1000), (3, 4097), (4, 4096), (2, 90), (2, 6000)])
 def test_paired_norm(device, dtype, n, C):
     from tessweave_engine_amd.kernels import ops
     g = torch.Generator().manual_seed(n)
@@ -172,6 +172,38 @@ def test_delta_rule_over_cut_sequences_in_reused_slots(device, H, G, D, E, most)
     assert (out.cpu().double() - want["c"]).abs().max() < 2e-5 * max(1.0, want["c"].abs().max().item())
 
 
+@pytest.mark.parametrize("H,G,D,E", [(2, 1, 64, 48), (1, 1, 128, 20), (2, 2, 200, 16)])
+def test_delta_rule_long_portions_solved_in_chunks(device, H, G, D, E):
+    """500 tokens in portions of 333 and 167 (neither a multiple of a chunk's 16 tokens) beside a second sequence of one
+    token a step: thirty chunks whose states follow from each other, slow decays, value columns in one to three blocks."""
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(D + E)
+    n = 500
+    W = 2 * G * D + H * E
+    rows, ab = torch.randn(n, W, generator=g), torch.randn(n, 2 * H, generator=g)
+    other, other_ab = torch.randn(2, W, generator=g), torch.randn(2, 2 * H, generator=g)
+    A_log, dt_bias = -2.0 + 0.5 * torch.randn(H, generator=g), -3.0 + torch.randn(H, generator=g)
+
+    def plain_of(r, gates):
+        return plain_delta_heads(r[:, :G * D].double(), r[:, G * D:2 * G * D].double(), r[:, 2 * G * D:].double(),
+                                 gates[:, :H].double(), gates[:, H:].double(), A_log.double(), dt_bias.double(), H, G, D, E)
+    want, want_other = plain_of(rows, ab), plain_of(other, other_ab)
+    state = torch.zeros(3, H, E, ops.delta_key_extent(D), device=device)
+    got, got_other, at = [], [], 0
+    for step, take in enumerate((333, 167)):
+        qkv = torch.cat([other[step:step + 1], rows[at:at + take]]).to(device)
+        gates = torch.cat([other_ab[step:step + 1], ab[at:at + take]]).to(device)
+        out = torch.full((take + 1, H * E), float("nan"), device=device)
+        ops.delta_rule(qkv, 0, G * D, 2 * G * D, gates, 0, H, A_log.to(device), dt_bias.to(device), state,
+                       ints([0, 1, take + 1], device), ints([2, 0], device), 0, 2, out, G, D, D ** -0.5, max_q_len=take)
+        got_other.append(out[:1].cpu())
+        got.append(out[1:].cpu())
+        at += take
+    for res, ref in ((torch.cat(got).double(), want), (torch.cat(got_other).double(), want_other)):
+        assert torch.isfinite(res).all()
+        assert (res - ref).abs().max() < 1e-4 * max(1.0, ref.abs().max().item()), (res - ref).abs().max()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_head_norm_with_gate(device, dtype):
     from tessweave_engine_amd.kernels import ops
@@ -186,14 +218,17 @@ def test_head_norm_with_gate(device, dtype):
     assert ((out.double().cpu() - want).abs() <= tol * (1 + want.abs())).all()
 
 
-def test_router_picks_the_largest_and_the_lowest_index_on_ties(device):
+@pytest.mark.parametrize("C,X,top", [(72, 70, 4), (90, 7, 3), (64, 1, 1), (2048, 16, 2)])
+def test_router_picks_the_largest_and_the_lowest_index_on_ties(device, C, X, top):
+    """Widths with and without 16-byte rows, an odd number of experts, one expert."""
     from tessweave_engine_amd.kernels import ops
     g = torch.Generator().manual_seed(2)
-    n, C, X, top = 40, 72, 70, 4
+    n = 40
     h = torch.randn(n, C, generator=g)
     router = torch.randn(X, C, generator=g) / math.sqrt(C)
-    router[5] = router[60]                                              # experts 5 and 60 always tie
-    router[9] = router[60] + 0.0
+    if X > 60:
+        router[5] = router[60]                                          # experts 5 and 60 always tie
+        router[9] = router[60] + 0.0
     ids = torch.empty(n, top, dtype=torch.int32, device=device)
     weights = torch.empty(n, top, device=device)
     ops.moe_route(h.to(device), router.to(device), top, ids, weights)
@@ -202,9 +237,9 @@ def test_router_picks_the_largest_and_the_lowest_index_on_ties(device):
         order = sorted(range(X), key=lambda e: (-round(z[t, e].item(), 9), e))
         chosen = ids[t].tolist()
         for e in chosen:
-            if e in (9, 60):
+            if X > 60 and e in (9, 60):
                 assert 5 in chosen and chosen.index(5) < chosen.index(e)
-        clear = [e for i, e in enumerate(order[:top]) if z[t, order[top]] < z[t, e] - 1e-4]
+        clear = [e for i, e in enumerate(order[:top]) if top == X or z[t, order[top]] < z[t, e] - 1e-4]
         assert set(clear) <= set(chosen)
         assert torch.allclose(weights[t].cpu().double(), torch.sigmoid(z[t, chosen]), atol=1e-5)
     # bfloat16 rows: the products are float32 of the rows as they are
@@ -215,7 +250,8 @@ def test_router_picks_the_largest_and_the_lowest_index_on_ties(device):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n,C,X,top,F", [(1, 88, 5, 2, 40), (9, 128, 16, 4, 64), (300, 96, 3, 3, 24), (130, 72, 64, 1, 100), (17, 64, 2, 1, 32)])
+@pytest.mark.parametrize("n,C,X,top,F", [(1, 88, 5, 2, 40), (9, 128, 16, 4, 64), (300, 96, 3, 3, 24), (130, 72, 64, 1, 100), (17, 64, 2, 1, 32),
+                                         (40, 64, 2, 1, 32), (7, 90, 6, 2, 40), (700, 256, 16, 2, 96)])
 def test_grouped_experts(device, dtype, n, C, X, top, F):
     """Against the plain expert, row by row, for given choices and scores (few rows, many rows an expert, experts
     nobody chose, sizes that are no multiples of 32); the result is added to what x held."""
