@@ -11,8 +11,12 @@
 // tile's expert's; combine (each token adds its experts' rows in the order it chose them). No launch waits for the
 // host, so the whole runs inside a captured graph.
 //
-// The experts' matrices lie stacked, row-major, with K padded to a multiple of 32 by zeros:
-//   gate, up [X][Fd][Cd], down [X][C][Fd]   (Fd, Cd: the inner size and the width rounded up to 32).
+// The experts' matrices lie stacked, K padded to a multiple of 32 by zeros and rows to a multiple of 16, in the order the
+// matrix unit's fragments are read: [X][rows / 16][K / (4 EPF)][piece 0..3][row 0..15][EPF] (EPF: the elements of 16
+// bytes), so that a wave's load of one fragment is 1 KB of consecutive memory (eight cache lines; row-major, its 16 rows
+// are 16 lines, and the loads queue for the cache's tag lookups):
+//   gate, up [X][Fd][Cd], down [X][C16][Fd]   (Fd, Cd: the inner size and the width rounded up to 32, C16: the width
+//   rounded up to 16). The gathered rows and the activations between the two products lie the same way.
 #include "gemm_shared.h"
 
 #define TW_MOE_MAX_EXPERTS 1024
@@ -163,14 +167,17 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const T* __restrict__ h
   const int row = blockIdx.x;
   if (tile_expert[row / TW_MOE_TILE] < 0) return;
   const int item = src_item[row];
-  T* dst = xs + (size_t)row * Cd;
+  constexpr int EPF = Elem<T>::kPerFrag;
+  // element c of the row: tile row / 16, step c / (4 EPF), piece c / EPF % 4, row row % 16 of the piece
+  T* dst = xs + (size_t)(row / TW_MOE_TILE) * Cd * TW_MOE_TILE + (row % TW_MOE_TILE) * EPF;
+  auto at = [](int c) { return (size_t)(c / EPF) * TW_MOE_TILE * EPF + c % EPF; };
   if (item < 0) {
-    for (int c = threadIdx.x; c < Cd; c += blockDim.x) dst[c] = tw_from_float<T>(0.f);
+    for (int c = threadIdx.x; c < Cd; c += blockDim.x) dst[at(c)] = tw_from_float<T>(0.f);
     return;
   }
   const float w = weights[item];
   const T* src = h + (size_t)(item / top) * ld_h;
-  for (int c = threadIdx.x; c < Cd; c += blockDim.x) dst[c] = tw_from_float<T>(c < C ? w * tw_to_float(src[c]) : 0.f);
+  for (int c = threadIdx.x; c < Cd; c += blockDim.x) dst[at(c)] = tw_from_float<T>(c < C ? w * tw_to_float(src[c]) : 0.f);
 }
 
 // ---- the grouped products ---------------------------------------------------------------------------------------
@@ -196,16 +203,19 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
   const int col0 = (SPLITK ? blockIdx.y : blockIdx.y * 4 + wave) * 16 * NT;
   if (col0 >= N) return;
   constexpr int KSTEP = 4 * EPF;
-  constexpr int k_stride = SPLITK ? 4 * KSTEP : KSTEP;
-  const int k_first = SPLITK ? wave * KSTEP : 0;
-  const T* a_ptr = A + (size_t)(tile * TW_MOE_TILE + r) * lda + g * EPF;
+  constexpr int BLK = 64 * EPF;                      // elements of one step's fragment of a tile: lane l's at l * EPF
+  constexpr int k_stride = (SPLITK ? 4 : 1) * BLK;    // (k counts the elements of a tile's fragments, step after step)
+  const int k_first = SPLITK ? wave * BLK : 0;
+  const size_t tile_elems = (size_t)K * TW_MOE_TILE;  // all steps of one tile of 16 rows
+  const int n_blocks = (N + 15) / 16;
+  const T* a_ptr = A + (size_t)tile * tile_elems + lane * EPF;
   const T* w_ptr[NT];
   const T* w2_ptr[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int col = min(col0 + t * 16 + r, N - 1);
-    w_ptr[t] = W + ((size_t)ex * N + col) * K + g * EPF;
-    w2_ptr[t] = GLU ? W2 + ((size_t)ex * N + col) * K + g * EPF : nullptr;
+    const size_t at = ((size_t)ex * n_blocks + min(col0 / 16 + t, n_blocks - 1)) * tile_elems + lane * EPF;
+    w_ptr[t] = W + at;
+    w2_ptr[t] = GLU ? W2 + at : nullptr;
   }
   f32x4 acc[MT][NT], acc2[MT][NT];
 #pragma unroll
@@ -219,7 +229,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int m = 0; m < MT; ++m) a[u][m] = tw_load_frag(a_ptr + (size_t)m * TW_MOE_TILE * lda + k + u * k_stride);
+      for (int m = 0; m < MT; ++m) a[u][m] = tw_load_frag(a_ptr + (size_t)m * tile_elems + k + u * k_stride);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         b[u][t] = tw_load_frag(w_ptr[t] + k + u * k_stride);
@@ -238,8 +248,9 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
   };
   constexpr int U = MT > 1 ? 2 : GLU ? 4 : (NT > 2 ? 4 : 8);
   int k = k_first;
-  for (; k + (U - 1) * k_stride < K; k += U * k_stride) steps(k, MoeCount<U>());
-  for (; k < K; k += k_stride) steps(k, MoeCount<1>());
+  const int k_end = (int)tile_elems;
+  for (; k + (U - 1) * k_stride < k_end; k += U * k_stride) steps(k, MoeCount<U>());
+  for (; k < k_end; k += k_stride) steps(k, MoeCount<1>());
   static_assert(!SPLITK || MT == 1);
   if constexpr (SPLITK) {
     __shared__ f32x4 part[GLU ? 2 : 1][3][NT][64];
@@ -268,9 +279,13 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
       if (col >= N) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const size_t at = (size_t)((tile + m) * TW_MOE_TILE + 4 * g + j) * ldo + col;
-        if (GLU) ((T*)out)[at] = tw_from_float<T>(tw_swish_limited(acc[m][t][j], acc2[m][t][j], limit));
-        else ((float*)out)[at] = acc[m][t][j];
+        if (GLU) {
+          // the activations are the next product's rows: in fragment order too (ldo: the elements of a row)
+          const size_t at = (size_t)(tile + m) * ldo * TW_MOE_TILE + ((size_t)(col / EPF) * TW_MOE_TILE + 4 * g + j) * EPF + col % EPF;
+          ((T*)out)[at] = tw_from_float<T>(tw_swish_limited(acc[m][t][j], acc2[m][t][j], limit));
+        } else {
+          ((float*)out)[(size_t)((tile + m) * TW_MOE_TILE + 4 * g + j) * ldo + col] = acc[m][t][j];
+        }
       }
     }
 }

@@ -1123,17 +1123,30 @@ def moe_pad(size):
     return (int(size) + 31) // 32 * 32
 
 
+def moe_blocked(w):
+    """Stacked matrices [X, N, K] (K a multiple of 32) in the order the grouped products read them: rows padded with zeros
+    to a multiple of 16, then [X, N16 / 16, K / (4 EPF), piece 0..3, row 0..15, EPF] (EPF: the elements of 16 bytes),
+    returned as [X, N16, K]: a wave's load of one fragment is 1 KB of consecutive memory."""
+    X, N, K = w.shape
+    epf = 16 // w.element_size()
+    _need(K % 32 == 0, "K must be padded to a multiple of 32")
+    N16 = (N + 15) // 16 * 16
+    if N16 != N:
+        w = torch.cat([w, w.new_zeros(X, N16 - N, K)], 1)
+    return w.reshape(X, N16 // 16, 16, K // (4 * epf), 4, epf).permute(0, 1, 3, 4, 2, 5).contiguous().reshape(X, N16, K)
+
+
 def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch):
     """x[n] += sum over a row's chosen experts e of down_e(glu(gate_e y, up_e y)), y = round(weights * h[n]), glu the
-    limited swish with LIMIT. gate, up [X, Fd, Cd], down [X, C, Fd] in h's type, zero padded (Fd, Cd: `moe_pad` of the
-    sizes). scratch(tag, shape, dtype) hands out the step's scratch tensors."""
+    limited swish with LIMIT. gate, up [X, Fd, Cd], down [X, C16, Fd] in h's type, zero padded (Fd, Cd: `moe_pad` of the
+    sizes, C16: C rounded up to 16) and laid out by `moe_blocked`. scratch(tag, shape, dtype) hands out the step's scratch tensors."""
     n, C, ld_h = _rows(h, "h")
     top = ids.shape[1]
     X, Fd, Cd = gate.shape
     _need(gate.is_contiguous() and up.is_contiguous() and down.is_contiguous() and gate.dtype == up.dtype == down.dtype == h.dtype,
           "the experts' matrices are contiguous and of h's type")
-    _need(tuple(up.shape) == (X, Fd, Cd) and tuple(down.shape) == (X, C, Fd) and Cd == moe_pad(C) and Fd % 32 == 0,
-          "the experts' matrices are [X, Fd, Cd] and [X, C, Fd]")
+    _need(tuple(up.shape) == (X, Fd, Cd) and tuple(down.shape) == (X, (C + 15) // 16 * 16, Fd) and Cd == moe_pad(C) and Fd % 32 == 0,
+          "the experts' matrices are [X, Fd, Cd] and [X, C16, Fd]")
     _need(ids.is_contiguous() and weights.is_contiguous() and tuple(ids.shape) == (n, top) and tuple(weights.shape) == (n, top),
           "ids and weights are [n, top]")
     nx, cx, ld_x = _rows(x, "x")

@@ -6,7 +6,8 @@
     expert(y) = down( g' * sigmoid(1.702 g') * (u' + 1) ),  g' = min(gate y, L),  u' = clamp(up y, -L, L)
 
 Experts have no biases. The experts' matrices are stacked on the device ([experts, inner, width] and [experts, width,
-inner], the reduction sizes padded to multiples of 32 with zeros) and all experts of a step run in two grouped
+inner], the reduction sizes padded to multiples of 32 with zeros, in the order the matrix unit's fragments are read:
+`ops.moe_blocked`) and all experts of a step run in two grouped
 products on the matrix unit, whose launch shapes depend on the step's rows only: nothing waits for the host.
 """
 from __future__ import annotations
@@ -59,7 +60,7 @@ class RoutedExperts(FeedForward):
             gate[e, :F, :C] = tensors.pop(g)
             up[e, :F, :C] = tensors.pop(u)
             down[e, :, :F] = tensors.pop(d)
-        self.gate, self.up, self.down = gate, up, down
+        self.gate, self.up, self.down = ops.moe_blocked(gate), ops.moe_blocked(up), ops.moe_blocked(down)
         if self.shared is not None:
             self.shared.bind(tensors, dtype, device)
 

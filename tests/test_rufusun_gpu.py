@@ -274,7 +274,8 @@ def test_grouped_experts(device, dtype, n, C, X, top, F):
     x0 = torch.randn(n, C, generator=g)
     x = x0.clone().to(device)
     ws = Workspace(device)
-    ops.moe_experts(h.to(device), ids.to(device), weights.to(device), gd.to(device), ud.to(device), dd.to(device), limit, x,
+    ops.moe_experts(h.to(device), ids.to(device), weights.to(device), ops.moe_blocked(gd.to(device)),
+                    ops.moe_blocked(ud.to(device)), ops.moe_blocked(dd.to(device)), limit, x,
                     lambda tag, shape, dtype: ws.get(tag, shape, dtype))
     want = x0.double().clone()
     for t in range(n):
