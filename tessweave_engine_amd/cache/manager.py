@@ -159,7 +159,7 @@ class CacheManager:
         # Live positions span at most window - 1 old keys plus one step's tokens;
         # such a span touches at most ceil(span / page) + 1 pages.
         span = spec.window - 1 + max(1, largest_step)
-        return min(full, math.ceil(span / self.page_size) + 1)
+        return min(full, math.ceil(span / self.page_size) + 1 + self.kept_blocks(group))
 
     def fits(self, total_tokens, largest_step):
         """Could a request of TOTAL_TOKENS ever be admitted (empty cache)?"""
@@ -233,6 +233,11 @@ class CacheManager:
             seq.block_keys = block_keys(tokens[:blocks * self.page_size], self.page_size, namespace, known=seq.block_keys)
         return seq.block_keys[:blocks]
 
+    def kept_blocks(self, group):
+        """Blocks at a request's start that a windowed GROUP never gives back (they hold its kept first tokens)."""
+        spec = self.layout.groups[group].spec
+        return math.ceil(spec.keep_first / self.page_size) if spec.window is not None else 0
+
     def first_needed_block(self, group, computed):
         """First logical block of GROUP that a query at position >= COMPUTED can see."""
         window = self.layout.groups[group].spec.window
@@ -283,7 +288,7 @@ class CacheManager:
                 continue
             table = seq.tables[g]
             first = min(self.first_needed_block(g, computed), len(table))
-            for b in range(first):
+            for b in range(self.kept_blocks(g), first):
                 if table[b] >= 0:
                     pool.release([table[b]])
                     table[b] = -1

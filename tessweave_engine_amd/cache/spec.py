@@ -13,11 +13,13 @@ from dataclasses import dataclass
 
 @dataclass(frozen=True)
 class PagedKV:
-    """Keys and values of every token (window None) or of the last `window` tokens."""
+    """Keys and values of every token (window None) or of the last `window` tokens; with a window, `keep_first` says
+    how many of a request's first tokens stay held whatever the window has passed."""
     kv_heads: int
     head_dim: int
     window: int | None = None
     value_dim: int | None = None      # size of a value if it differs from a key's (None: head_dim)
+    keep_first: int = 0
 
     def __post_init__(self):
         if self.value_dim == self.head_dim:
@@ -26,6 +28,10 @@ class PagedKV:
             raise ValueError("kv_heads, head_dim and value_dim must be positive")
         if self.window is not None and self.window <= 0:
             raise ValueError("a window must be positive (None means all keys)")
+        if self.keep_first < 0:
+            raise ValueError("keep_first cannot be negative")
+        if self.window is None:
+            object.__setattr__(self, "keep_first", 0)          # (without a window everything is kept anyway)
 
 
 @dataclass(frozen=True)

@@ -4,7 +4,8 @@
 //   values [pages][kv_heads][E][page_size]     (transposed inside a page; E may differ from D)
 //
 // For query position i and key position j of one sequence (0 <= i - j < window, or every j <= i
-// without a window):
+// without a window; with a window, the first `keep` keys of the sequence stay visible to every later query, at
+// their true positions):
 //   raw_g(i, j)  = scale * q_ig . k_j,kv(g) - slope_g * (i - j)            (slopes optional)
 //   s_h(i, j)    = sum_g talk[h][g] * raw_g(i, j)                          (talk optional: s = raw)
 //   p_h(i, j)    = exp(s_h(i, j)) / (exp(sink_h) + sum_j' exp(s_h(i, j')))   (sink optional)
@@ -46,6 +47,7 @@ struct MixedAttnArgs {
   float* part;                       // splits > 1: [seq - seq0][tile][split][H][rows_kept][E + 2] (output sums, max, sum)
   float scale, out_scale;
   int H, G, D, E, P, window, splits;
+  int keep;                          // with a window: keys 0 .. keep - 1 are seen by every later query as well
   int page_shift;                    // log2(P) if P is a power of two, else -1
   int rows_kept;                     // rows of a tile whose partial results are kept: 1 for one-token sequences, else 16
   int q_in_lds;                      // 0: the tile's queries do not fit LDS beside the raw scores; fragments are read from memory
@@ -113,12 +115,19 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   // ---- the key tiles of this workgroup ---------------------------------------------------------------------
   const int lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;       // first key any row of the tile sees
   const int hi = pos0 + n_rows - 1;                                     // last key (its own position)
-  int tile_lo = lo / 16, tile_hi = hi / 16 + 1;
+  // The key tiles a workgroup walks are numbered without the gap between the kept first keys and the window: tiles
+  // 0 .. kept - 1 hold the kept keys that lie before the window's first tile, the tiles behind them are the window's.
+  const int keep = a.window > 0 ? a.keep : 0;
+  const int win_lo = lo / 16;
+  const int kept = min((keep + 15) / 16, win_lo);
+  const int skip = win_lo - kept;                                        // key tile of walk index v >= kept: v + skip
+  int tile_lo = 0, tile_hi = hi / 16 + 1 - skip;
   if (a.splits > 1) {
     const int per = (tile_hi - tile_lo + a.splits - 1) / a.splits;
     tile_lo = tile_lo + blockIdx.z * per;
     tile_hi = min(tile_hi, tile_lo + per);
   }
+  auto key_tile = [&](int v) { return v < kept ? v : v + skip; };
   const bool with_sink = a.sink != nullptr && (a.splits == 1 || blockIdx.z == 0);
 
   float m[HPW], l[HPW];
@@ -155,17 +164,17 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   const int shift = a.page_shift;
   auto page_of = [&](int p) { return shift >= 0 ? p >> shift : p / P; };
   auto in_page = [&](int p) { return shift >= 0 ? p & (P - 1) : p % P; };
-  auto key_page = [&](int kt) -> int {
-    const int p = kt * 16 + r;
-    return (kt < tile_hi && p < kv_len && p >= lo) ? table[page_of(p)] : -1;
+  auto key_page = [&](int v) -> int {
+    const int p = key_tile(v) * 16 + r;
+    return (v < tile_hi && p < kv_len && (p >= lo || p < keep)) ? table[page_of(p)] : -1;
   };
-  auto value_page = [&](int kt) -> int {
-    const int p = kt * 16 + 4 * g;
-    return (kt < tile_hi && p < kv_len && p + 3 >= lo) ? table[page_of(p)] : -1;
+  auto value_page = [&](int v) -> int {
+    const int p = key_tile(v) * 16 + 4 * g;
+    return (v < tile_hi && p < kv_len && (p + 3 >= lo || p < keep)) ? table[page_of(p)] : -1;
   };
-  auto request_keys = [&](int kt, int page) {
+  auto request_keys = [&](int v, int page) {
     if constexpr (!AHEAD) return;
-    const int p = kt * 16 + r;
+    const int p = key_tile(v) * 16 + r;
 #pragma unroll
     for (int i = 0; i < KVN; ++i) {
       const int head = wave * HPW + i;                     // (SHARE: the wave's first head stands for all)
@@ -184,10 +193,10 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   int vpage = value_page(tile_lo);
   int buf = 0;
   for (int kt = tile_lo; kt < tile_hi; ++kt, buf ^= 1) {
-    const int p0 = kt * 16;
+    const int p0 = key_tile(kt) * 16;
     // A tile whose 16 keys every row of the query tile sees (none beyond the first row's position, none before
     // the last row's window) needs no masks; most tiles of a long window are such.
-    const bool interior = p0 + 15 <= pos0 && (a.window == 0 || p0 >= pos0 + n_rows - a.window);
+    const bool interior = p0 + 15 <= pos0 && (a.window == 0 || p0 >= pos0 + n_rows - a.window || p0 + 15 < keep);
     // ---- raw scores of this wave's heads ---------------------------------------------------------------
     f32x4 raw_own[HPW];
     {
@@ -274,7 +283,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int p = p0 + 4 * g + e;
-            const bool ok = p < kv_len && p <= t_row && p >= lo_row;
+            const bool ok = p < kv_len && p <= t_row && (p >= lo_row || p < keep);
             s[e] = ok ? s[e] : -INFINITY;
           }
         }
@@ -303,7 +312,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
             if (!interior) {
 #pragma unroll
               for (int e = 0; e < 4; ++e)
-                if (pv + e >= kv_len || pv + e < lo) v[e] = tw_from_float<T>(0.f);
+                if (pv + e >= kv_len || (pv + e < lo && pv + e >= keep)) v[e] = tw_from_float<T>(0.f);
             }
             if (rescale) {
 #pragma unroll
@@ -453,9 +462,9 @@ extern "C" int tw_attn_mixed(int dtype, const void* q, long ldq, const void* key
                              int seq0, int n_seqs, int max_q_len, void* out, long ldo, const float* talk,
                              const float* sink, const float* slopes, float* workspace, long workspace_floats,
                              int q_heads, int kv_heads, int key_dim, int value_dim, int page_size, int window,
-                             float scale, float out_scale, int splits, hipStream_t stream) {
+                             int keep_first, float scale, float out_scale, int splits, hipStream_t stream) {
   TW_REQUIRE(q && keys && values && block_table && q_start && kv_len && out);
-  TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && max_q_len >= 1 && splits >= 1 && window >= 0);
+  TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && max_q_len >= 1 && splits >= 1 && window >= 0 && keep_first >= 0);
   TW_REQUIRE(q_heads >= 1 && q_heads <= 32 && kv_heads >= 1 && q_heads % kv_heads == 0);
   TW_REQUIRE(key_dim % 16 == 0 && key_dim >= 16 && key_dim <= 256 && value_dim % 16 == 0 && value_dim >= 16 && value_dim <= 256);
   TW_REQUIRE(page_size > 0 && page_size % 4 == 0);
@@ -469,7 +478,7 @@ extern "C" int tw_attn_mixed(int dtype, const void* q, long ldq, const void* key
   }
   if (n_seqs == 0) return 0;
   MixedAttnArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, seq0, out, ldo, talk, sink, slopes,
-                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits, -1, 16, 1};
+                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits, keep_first, -1, 16, 1};
   if (dtype == TW_DTYPE_BF16) return mixed_dispatch<bf16_t>(a, n_seqs, max_q_len, stream);
   if (dtype == TW_DTYPE_F32) return mixed_dispatch<float>(a, n_seqs, max_q_len, stream);
   return TW_ERR_BAD_ARGUMENT;

@@ -419,7 +419,8 @@ extern "C" int tw_delta_rule(const float* qkv, long ld_qkv, int q_col, int k_col
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, long ld_o, const float* __restrict__ gate,
                                                              long ld_g, const float* __restrict__ weight, T* __restrict__ out,
-                                                             long ld_out, int n, int H, int E, float eps) {
+                                                             long ld_out, int n, int H, int E, float eps, int weight_stride,
+                                                             int gate_kind) {
   const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (unit >= n * H) return;
   const int lane = threadIdx.x & 63;
@@ -433,20 +434,24 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   T* dst = out + (size_t)row * ld_out + (size_t)head * E;
   for (int e = lane; e < E; e += 64) {
     const float z = g[e];
-    dst[e] = tw_from_float<T>(src[e] * rinv * weight[e] * (z / (1.f + expf(-z))));
+    const float sig = 1.f / (1.f + expf(-z));
+    // weight_stride: 0 for one weight vector for all heads, E for one a head; gate_kind 0: SiLU of the gate, 1: its sigmoid
+    dst[e] = tw_from_float<T>(src[e] * rinv * weight[(size_t)head * weight_stride + e] * (gate_kind == 1 ? sig : z * sig));
   }
 }
 
 extern "C" int tw_head_norm_gate(int dtype, const float* o, long ld_o, const float* gate, long ld_g, const float* weight,
-                                 void* out, long ld_out, int n, int H, int E, float eps, hipStream_t stream) {
-  TW_REQUIRE(o && gate && weight && out && n >= 0 && H > 0 && E > 0 && eps > 0.f);
+                                 void* out, long ld_out, int n, int H, int E, float eps, int weight_per_head, int gate_kind,
+                                 hipStream_t stream) {
+  TW_REQUIRE(o && gate && weight && out && n >= 0 && H > 0 && E > 0 && eps > 0.f && (gate_kind == 0 || gate_kind == 1));
+  const int weight_stride = weight_per_head ? E : 0;
   TW_REQUIRE(ld_o >= (long)H * E && ld_g >= (long)H * E && ld_out >= (long)H * E);
   if (n == 0) return 0;
   const int blocks = tw_div_up((long)n * H, 4);
   if (dtype == TW_DTYPE_BF16)
-    head_norm_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(o, ld_o, gate, ld_g, weight, (bf16_t*)out, ld_out, n, H, E, eps);
+    head_norm_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(o, ld_o, gate, ld_g, weight, (bf16_t*)out, ld_out, n, H, E, eps, weight_stride, gate_kind);
   else if (dtype == TW_DTYPE_F32)
-    head_norm_gate_kernel<float><<<blocks, 256, 0, stream>>>(o, ld_o, gate, ld_g, weight, (float*)out, ld_out, n, H, E, eps);
+    head_norm_gate_kernel<float><<<blocks, 256, 0, stream>>>(o, ld_o, gate, ld_g, weight, (float*)out, ld_out, n, H, E, eps, weight_stride, gate_kind);
   else return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
 }

@@ -4,6 +4,11 @@
 //   out = sum over the chosen experts e of  expert_e(s_e * h)         (the score multiplies the expert's INPUT)
 //   expert(y): down( glu(gate y, up y) ), glu as TW_GLU_SWISH_LIMITED with the experts' limit
 //
+// A second kind of expert and of weighting (`kind` 1 of tw_moe_experts, `mode` 1 of tw_moe_route):
+//   z = W_router h + b        chosen: the `top` largest      p = softmax over the chosen logits alone
+//   out = sum over the chosen experts e of  p_e * expert_e(h)         (the weight multiplies the expert's OUTPUT)
+//   expert(y): down( gelu(up y) ), the exact gelu y Phi(y); no gate matrix
+//
 // A step runs in six launches whose shapes depend only on the number of rows: route; plan (every expert's rows are
 // laid out one expert after the other, each expert's share padded to whole tiles of 16 rows; which expert a tile
 // belongs to is a table on the device, tiles nobody uses say -1); gather (the scaled, rounded input rows in that
@@ -27,8 +32,8 @@
 // ---- route ---------------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, long ld_h, const float* __restrict__ router,
-                                                        int C, int X, int top, int* __restrict__ ids,
-                                                        float* __restrict__ weights) {
+                                                        const float* __restrict__ bias, int mode, int C, int X, int top,
+                                                        int* __restrict__ ids, float* __restrict__ weights) {
   __shared__ float z[TW_MOE_MAX_EXPERTS];
   const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* x = h + (size_t)row * ld_h;
@@ -63,8 +68,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     s0 = tw_wave_sum(s0);
     s1 = tw_wave_sum(s1);
     if (lane == 0) {
-      z[e] = s0;
-      if (e + 1 < X) z[e + 1] = s1;
+      z[e] = s0 + (bias ? bias[e] : 0.f);
+      if (e + 1 < X) z[e + 1] = s1 + (bias ? bias[e + 1] : 0.f);
     }
   }
   __syncthreads();
@@ -84,23 +89,34 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     }
     if (lane == 0) {
       ids[(size_t)row * top + r] = at;
-      weights[(size_t)row * top + r] = 1.f / (1.f + expf(-best));
+      weights[(size_t)row * top + r] = mode == 1 ? best : 1.f / (1.f + expf(-best));
       z[at] = -INFINITY;
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
   }
+  if (mode == 1 && lane == 0) {
+    // the softmax over the chosen logits alone (the first chosen is the largest), in the order they were chosen
+    float* w = weights + (size_t)row * top;
+    const float first = w[0];
+    float sum = 0.f;
+    for (int r = 0; r < top; ++r) {
+      w[r] = expf(w[r] - first);
+      sum += w[r];
+    }
+    for (int r = 0; r < top; ++r) w[r] = w[r] / sum;
+  }
 }
 
-extern "C" int tw_moe_route(int dtype, const void* h, long ld_h, const float* router, int n, int C, int X, int top, int* ids,
-                            float* weights, hipStream_t stream) {
-  TW_REQUIRE(h && router && ids && weights && n >= 0 && C > 0 && ld_h >= C);
+extern "C" int tw_moe_route(int dtype, const void* h, long ld_h, const float* router, const float* bias, int mode, int n, int C,
+                            int X, int top, int* ids, float* weights, hipStream_t stream) {
+  TW_REQUIRE(h && router && ids && weights && n >= 0 && C > 0 && ld_h >= C && (mode == 0 || mode == 1));
   TW_REQUIRE(X > 0 && X <= TW_MOE_MAX_EXPERTS && top > 0 && top <= X);
   if (n == 0) return 0;
   if (dtype == TW_DTYPE_BF16)
-    moe_route_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)h, ld_h, router, C, X, top, ids, weights);
+    moe_route_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)h, ld_h, router, bias, mode, C, X, top, ids, weights);
   else if (dtype == TW_DTYPE_F32)
-    moe_route_kernel<float><<<n, 256, 0, stream>>>((const float*)h, ld_h, router, C, X, top, ids, weights);
+    moe_route_kernel<float><<<n, 256, 0, stream>>>((const float*)h, ld_h, router, bias, mode, C, X, top, ids, weights);
   else return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
 }
@@ -175,7 +191,7 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const T* __restrict__ h
     for (int c = threadIdx.x; c < Cd; c += blockDim.x) dst[at(c)] = tw_from_float<T>(0.f);
     return;
   }
-  const float w = weights[item];
+  const float w = weights ? weights[item] : 1.f;          // (no weights: they multiply the experts' outputs instead)
   const T* src = h + (size_t)(item / top) * ld_h;
   for (int c = threadIdx.x; c < Cd; c += blockDim.x) dst[at(c)] = tw_from_float<T>(c < C ? w * tw_to_float(src[c]) : 0.f);
 }
@@ -190,11 +206,14 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const T* __restrict__ h
 // MT > 1 (steps of many rows, whose experts' shares are padded to MT tiles): a workgroup takes MT tiles of one expert
 // against every fragment of the expert's matrices it reads.
 template <int N> struct MoeCount { static constexpr int value = N; };
-template <typename T, bool GLU, int NT, bool SPLITK = false, int MT = 1>
+// ACT 0: the float32 product; 1: gate and up with the limited swish; 2: one matrix with the exact gelu (1 and 2 write the
+// next product's rows in the compute type).
+template <typename T, int ACT, int NT, bool SPLITK = false, int MT = 1>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ A, long lda, const T* __restrict__ W,
                                                           const T* __restrict__ W2, const int* __restrict__ tile_expert,
                                                           void* __restrict__ out, long ldo, int N, int K, float limit) {
   constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr bool GLU = ACT == 1;
   const int tile = blockIdx.x * MT;
   const int ex = tile_expert[tile];
   if (ex < 0) return;
@@ -279,10 +298,12 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
       if (col >= N) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (GLU) {
+        if (ACT != 0) {
           // the activations are the next product's rows: in fragment order too (ldo: the elements of a row)
           const size_t at = (size_t)(tile + m) * ldo * TW_MOE_TILE + ((size_t)(col / EPF) * TW_MOE_TILE + 4 * g + j) * EPF + col % EPF;
-          ((T*)out)[at] = tw_from_float<T>(tw_swish_limited(acc[m][t][j], acc2[m][t][j], limit));
+          const float z = acc[m][t][j];
+          ((T*)out)[at] = tw_from_float<T>(GLU ? tw_swish_limited(z, acc2[m][t][j], limit)
+                                               : 0.5f * z * (1.f + erff(z * 0.70710678118654752f)));
         } else {
           ((float*)out)[(size_t)((tile + m) * TW_MOE_TILE + 4 * g + j) * ldo + col] = acc[m][t][j];
         }
@@ -292,22 +313,31 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
 
 // ---- combine: x[token] += its experts' rows, in the order of its choices ------------------------------------------
 // A workgroup takes 1,024 columns of a row, four a thread where rows and addresses allow 16-byte accesses.
+// weights (or null): a factor on each of the token's rows; accumulate 0: x is written, not added to.
 template <bool VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long ld_x, const float* __restrict__ ys,
-                                                          long ld_y, const int* __restrict__ pos, int C, int top) {
+                                                          long ld_y, const int* __restrict__ pos, int C, int top,
+                                                          const float* __restrict__ weights, int accumulate) {
   const int row = blockIdx.x;
   const int c = blockIdx.y * 1024 + threadIdx.x * 4;
   if (c >= C) return;
   if constexpr (VEC) {
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (int r = 0; r < top; ++r) sum += *reinterpret_cast<const f32x4*>(ys + (size_t)pos[(size_t)row * top + r] * ld_y + c);
+    for (int r = 0; r < top; ++r) {
+      const f32x4 y = *reinterpret_cast<const f32x4*>(ys + (size_t)pos[(size_t)row * top + r] * ld_y + c);
+      if (weights) sum += weights[(size_t)row * top + r] * y;
+      else sum += y;
+    }
     f32x4* dst = reinterpret_cast<f32x4*>(x + (size_t)row * ld_x + c);
-    *dst += sum;
+    if (accumulate) *dst += sum;
+    else *dst = sum;
   } else {
     for (int j = 0; j < 4 && c + j < C; ++j) {
       float sum = 0.f;
-      for (int r = 0; r < top; ++r) sum += ys[(size_t)pos[(size_t)row * top + r] * ld_y + c + j];
-      x[(size_t)row * ld_x + c + j] += sum;
+      for (int r = 0; r < top; ++r)
+        sum += (weights ? weights[(size_t)row * top + r] : 1.f) * ys[(size_t)pos[(size_t)row * top + r] * ld_y + c + j];
+      if (accumulate) x[(size_t)row * ld_x + c + j] += sum;
+      else x[(size_t)row * ld_x + c + j] = sum;
     }
   }
 }
@@ -318,8 +348,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
 extern "C" int tw_moe_experts(int dtype, const void* h, long ld_h, const int* ids, const float* weights, int n, int top, int X,
                               const void* gate, const void* up, const void* down, int C, int Cd, int Fd, float limit,
                               int* pos, int* src_item, int* tile_expert, void* xs, void* act, float* ys, int capacity,
-                              float* x, long ld_x, hipStream_t stream) {
-  TW_REQUIRE(h && ids && weights && gate && up && down && pos && src_item && tile_expert && xs && act && ys && x);
+                              float* x, long ld_x, int kind, int accumulate, hipStream_t stream) {
+  TW_REQUIRE(h && ids && weights && up && down && pos && src_item && tile_expert && xs && act && ys && x);
+  TW_REQUIRE((kind == 0 && gate) || kind == 1);
+  if (kind == 1) gate = up;            // (never read: the alignment test below wants a pointer)
   TW_REQUIRE(n >= 0 && top > 0 && C > 0 && Cd >= C && Cd % 32 == 0 && Fd > 0 && Fd % 32 == 0 && ld_h >= C && ld_x >= C);
   TW_REQUIRE((uintptr_t)xs % 16 == 0 && (uintptr_t)act % 16 == 0 && (uintptr_t)gate % 16 == 0 && (uintptr_t)up % 16 == 0 &&
              (uintptr_t)down % 16 == 0);
@@ -336,40 +368,66 @@ extern "C" int tw_moe_experts(int dtype, const void* h, long ld_h, const int* id
   const dim3 glu_wide(tiles / TW_MOE_WIDE, tw_div_up(Fd, 4 * 16 * 2)), down_wide(tiles / TW_MOE_WIDE, tw_div_up(C, 4 * 16 * 2));
   if (dtype == TW_DTYPE_BF16) {
     typedef bf16_t T;
-    moe_gather_kernel<T><<<capacity, 256, 0, stream>>>((const T*)h, ld_h, weights, src_item, tile_expert, (T*)xs, C, Cd, top);
+    moe_gather_kernel<T><<<capacity, 256, 0, stream>>>((const T*)h, ld_h, kind == 0 ? weights : nullptr, src_item, tile_expert,
+                                                       (T*)xs, C, Cd, top);
     if (few) {
-      moe_grouped_kernel<T, true, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
-                                                                        tile_expert, act, Fd, Fd, Cd, limit);
-      moe_grouped_kernel<T, false, 2, true><<<down_few, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+      if (kind == 0)
+        moe_grouped_kernel<T, 1, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                       tile_expert, act, Fd, Fd, Cd, limit);
+      else
+        moe_grouped_kernel<T, 2, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)up, nullptr,
+                                                                       tile_expert, act, Fd, Fd, Cd, 0.f);
+      moe_grouped_kernel<T, 0, 2, true><<<down_few, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
                                                                          tile_expert, ys, C, C, Fd, 0.f);
     } else if (wide) {
-      moe_grouped_kernel<T, true, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
-          (const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert, act, Fd, Fd, Cd, limit);
-      moe_grouped_kernel<T, false, 2, false, TW_MOE_WIDE><<<down_wide, 256, 0, stream>>>(
+      if (kind == 0)
+        moe_grouped_kernel<T, 1, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
+            (const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert, act, Fd, Fd, Cd, limit);
+      else
+        moe_grouped_kernel<T, 2, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
+            (const T*)xs, Cd, (const T*)up, nullptr, tile_expert, act, Fd, Fd, Cd, 0.f);
+      moe_grouped_kernel<T, 0, 2, false, TW_MOE_WIDE><<<down_wide, 256, 0, stream>>>(
           (const T*)act, Fd, (const T*)down, nullptr, tile_expert, ys, C, C, Fd, 0.f);
     } else {
-      moe_grouped_kernel<T, true, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
-                                                                   tile_expert, act, Fd, Fd, Cd, limit);
-      moe_grouped_kernel<T, false, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+      if (kind == 0)
+        moe_grouped_kernel<T, 1, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                  tile_expert, act, Fd, Fd, Cd, limit);
+      else
+        moe_grouped_kernel<T, 2, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)up, nullptr,
+                                                                  tile_expert, act, Fd, Fd, Cd, 0.f);
+      moe_grouped_kernel<T, 0, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
                                                                     tile_expert, ys, C, C, Fd, 0.f);
     }
   } else if (dtype == TW_DTYPE_F32) {
     typedef float T;
-    moe_gather_kernel<T><<<capacity, 256, 0, stream>>>((const T*)h, ld_h, weights, src_item, tile_expert, (T*)xs, C, Cd, top);
+    moe_gather_kernel<T><<<capacity, 256, 0, stream>>>((const T*)h, ld_h, kind == 0 ? weights : nullptr, src_item, tile_expert,
+                                                       (T*)xs, C, Cd, top);
     if (few) {
-      moe_grouped_kernel<T, true, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
-                                                                        tile_expert, act, Fd, Fd, Cd, limit);
-      moe_grouped_kernel<T, false, 2, true><<<down_few, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+      if (kind == 0)
+        moe_grouped_kernel<T, 1, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                       tile_expert, act, Fd, Fd, Cd, limit);
+      else
+        moe_grouped_kernel<T, 2, 2, true><<<glu_few, 256, 0, stream>>>((const T*)xs, Cd, (const T*)up, nullptr,
+                                                                       tile_expert, act, Fd, Fd, Cd, 0.f);
+      moe_grouped_kernel<T, 0, 2, true><<<down_few, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
                                                                          tile_expert, ys, C, C, Fd, 0.f);
     } else if (wide) {
-      moe_grouped_kernel<T, true, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
-          (const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert, act, Fd, Fd, Cd, limit);
-      moe_grouped_kernel<T, false, 2, false, TW_MOE_WIDE><<<down_wide, 256, 0, stream>>>(
+      if (kind == 0)
+        moe_grouped_kernel<T, 1, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
+            (const T*)xs, Cd, (const T*)gate, (const T*)up, tile_expert, act, Fd, Fd, Cd, limit);
+      else
+        moe_grouped_kernel<T, 2, 2, false, TW_MOE_WIDE><<<glu_wide, 256, 0, stream>>>(
+            (const T*)xs, Cd, (const T*)up, nullptr, tile_expert, act, Fd, Fd, Cd, 0.f);
+      moe_grouped_kernel<T, 0, 2, false, TW_MOE_WIDE><<<down_wide, 256, 0, stream>>>(
           (const T*)act, Fd, (const T*)down, nullptr, tile_expert, ys, C, C, Fd, 0.f);
     } else {
-      moe_grouped_kernel<T, true, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
-                                                                   tile_expert, act, Fd, Fd, Cd, limit);
-      moe_grouped_kernel<T, false, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
+      if (kind == 0)
+        moe_grouped_kernel<T, 1, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)gate, (const T*)up,
+                                                                  tile_expert, act, Fd, Fd, Cd, limit);
+      else
+        moe_grouped_kernel<T, 2, 2><<<glu_grid, 256, 0, stream>>>((const T*)xs, Cd, (const T*)up, nullptr,
+                                                                  tile_expert, act, Fd, Fd, Cd, 0.f);
+      moe_grouped_kernel<T, 0, 4><<<down_grid, 256, 0, stream>>>((const T*)act, Fd, (const T*)down, nullptr,
                                                                     tile_expert, ys, C, C, Fd, 0.f);
     }
   } else {
@@ -377,8 +435,8 @@ extern "C" int tw_moe_experts(int dtype, const void* h, long ld_h, const int* id
   }
   const dim3 combine_grid(n, tw_div_up(C, 1024));
   if (C % 4 == 0 && ld_x % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)ys % 16 == 0)
-    moe_combine_kernel<true><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top);
+    moe_combine_kernel<true><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top, kind == 1 ? weights : nullptr, accumulate);
   else
-    moe_combine_kernel<false><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top);
+    moe_combine_kernel<false><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top, kind == 1 ? weights : nullptr, accumulate);
   return TW_LAUNCH_RESULT();
 }

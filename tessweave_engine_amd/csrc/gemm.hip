@@ -768,7 +768,7 @@ extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const 
 extern "C" int tw_linear_act(int dtype, const void* A, long lda, const void* W, long ldw, int shuffled, const float* bias,
                              void* C, long ldc, float* partial, long partial_bytes, int M, int N, int K, int act,
                              hipStream_t stream) {
-  TW_REQUIRE(act == TW_ACT_RELU_SQUARED);
+  TW_REQUIRE(act == TW_ACT_RELU_SQUARED || act == TW_ACT_GELU_ERF);
   TW_REQUIRE(M > 64 && N > 0 && K > 0 && lda >= K && ldc >= N && K % (dtype == TW_DTYPE_F32 ? 4 : 8) == 0);
   TW_REQUIRE(dtype == TW_DTYPE_F32 || dtype == TW_DTYPE_BF16);
   TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K));

@@ -37,14 +37,16 @@ __device__ __forceinline__ float tw_glu(float g, float u, long code) {
 }
 
 // A plain product that adds no residual has the residual's row stride free as well: there it names an activation
-// of the result (after the bias, before the one rounding). 0: none; TW_ACT_RELU_SQUARED: max(x, 0)^2. Only the tiled
+// of the result (after the bias, before the one rounding). 0: none; TW_ACT_RELU_SQUARED: max(x, 0)^2; TW_ACT_GELU_ERF. Only the tiled
 // kernels (and the reduction of their split-K sums) read it: tw_linear_act is the entry point.
 #define TW_ACT_RELU_SQUARED 1
+#define TW_ACT_GELU_ERF 2          /* the exact gelu, x Phi(x) */
 __device__ __forceinline__ float tw_act(float x, long code) {
   if (code == TW_ACT_RELU_SQUARED) {
     x = fmaxf(x, 0.f);
     return x * x;
   }
+  if (code == TW_ACT_GELU_ERF) return 0.5f * x * (1.f + erff(x * 0.70710678118654752f));
   return x;
 }
 

@@ -328,6 +328,7 @@ struct LatentDecodeArgs {
   float* part;
   float scale;
   int H, K, Lp, P, splits;
+  const float* sink;                  // [H] or null: exp(sink_a) more in head a's denominator (no key, no value, not scaled)
 };
 
 template <typename T> __device__ __forceinline__ float lt_exp(float v);
@@ -452,6 +453,13 @@ __global__ __launch_bounds__(256) void latent_decode_kernel(LatentDecodeArgs a) 
       total += f * sw[w * 16 + hh];
     }
     if (a.splits == 1) {
+      if (a.sink) {
+        const float sk = a.sink[ht * 16 + hh];
+        const float both = fmaxf(top, sk);
+        const float f = top == -INFINITY ? 0.f : lt_exp<T>(top - both);
+        o *= f;
+        total = total * f + lt_exp<T>(sk - both);
+      }
       ((T*)a.out)[(size_t)row * a.ldo + (size_t)(ht * 16 + hh) * Lp + l] = tw_from_float<T>(o / total);
     } else {
       float* dst = a.part + ((((size_t)s * gridDim.z + ht) * a.splits + split) * 16 + hh) * (Lp + 2);
@@ -479,11 +487,13 @@ __global__ __launch_bounds__(256) void latent_decode_merge_kernel(LatentDecodeAr
   if (threadIdx.x < 64) {
     const int sp = threadIdx.x;
     const float m = sp < a.splits ? base[sp * stride + Lp] : -INFINITY;
-    const float top = tw_wave_max(m);
+    float top = tw_wave_max(m);
+    const float sk = a.sink ? a.sink[head] : -INFINITY;
+    top = fmaxf(top, sk);
     const float f = m == -INFINITY ? 0.f : lt_exp<T>(m - top);
     weight[sp] = f;
     const float total = tw_wave_sum(sp < a.splits ? f * base[sp * stride + Lp + 1] : 0.f);
-    if (sp == 0) total_s = total;
+    if (sp == 0) total_s = total + (a.sink ? lt_exp<T>(sk - top) : 0.f);
   }
   __syncthreads();
   const float inv = 1.f / total_s;
@@ -511,7 +521,7 @@ extern "C" long tw_latent_decode_workspace_floats(int n_seqs, int heads, int Lp,
 extern "C" int tw_latent_decode(int dtype, const void* q, long ldq, const void* keys, const void* values,
                                 const int* block_table, int table_stride, const int* q_start, const int* kv_len,
                                 int n_seqs, void* out, long ldo, float* workspace, long workspace_floats, int heads,
-                                int K, int Lp, int page_size, float scale, int splits, hipStream_t stream) {
+                                int K, int Lp, int page_size, float scale, int splits, const float* sink, hipStream_t stream) {
   TW_REQUIRE(q && keys && values && block_table && q_start && kv_len && out && n_seqs >= 0 && splits >= 1 && splits <= 64);
   TW_REQUIRE(heads >= 1 && K % 16 == 0 && K <= 256 && Lp % 16 == 0 && Lp >= 16 && Lp <= 240 && Lp <= K);
   TW_REQUIRE(page_size > 0 && page_size % 4 == 0);
@@ -521,7 +531,7 @@ extern "C" int tw_latent_decode(int dtype, const void* q, long ldq, const void* 
   if (splits > 1) TW_REQUIRE(workspace && workspace_floats >= tw_latent_decode_workspace_floats(n_seqs, heads, Lp, splits));
   if (n_seqs == 0) return 0;
   LatentDecodeArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, out, ldo, workspace, scale,
-                     heads, K, Lp, page_size, splits};
+                     heads, K, Lp, page_size, splits, sink};
   const int head_tiles = tw_div_up(heads, 16);
   const dim3 grid(n_seqs, splits, head_tiles);
   const size_t lds = ((size_t)4 * 16 * (Lp + 4) + 128) * sizeof(float);

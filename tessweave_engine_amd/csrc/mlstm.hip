@@ -1,0 +1,303 @@
+// The matrix memory of the mLSTM: per head a state S [D][E], a normaliser n [D] and a running maximum m of the gates'
+// logarithms, all float32 and all zero (m too) when a request opens. Per token, with the log input gate i and the log
+// forget gate f (both capped: i = cap tanh(z_i / cap), f = logsigmoid(cap tanh(z_f / cap))):
+//
+//   m' = max(f + m, i);  S <- exp(f + m - m') S + exp(i - m') k v^T;  n likewise with k alone;
+//   o = S^T q / (max(|n . q|, exp(-m')) + 1e-6)
+//
+// q, k, v and the gates' raw values come as float32 rows of one packed product; everything here is float32.
+// State layout: S [requests][H][Ep][Dp] (a value column's keys are contiguous; Dp, Ep: D and E rounded up to 16, the
+// tails are zeros), n [requests][2][H][Dp] and m [requests][2][H] held twice: a step reads copy phase[s] and writes the
+// other (several workgroups of a head read n and m while one of them writes).
+//
+// mlstm_walk: sequences of a few tokens, token by token. A workgroup owns 16 value columns of one (sequence, head);
+// lane 16 c + s keeps the keys s, s + 16, .. of column c (and of n) in registers; a token's two products are a few
+// multiply-adds and a sum over 16 neighbouring lanes.
+//
+// mlstm_chunk: longer portions, 16 tokens at once on the matrix unit (float32 products). With F_t the running sum of
+// f inside the chunk, u_j = i_j - F_j, g_t = max(m0, max_{j <= t} u_j) and m_t = F_t + g_t:
+//   o_t  = [ exp(m0 - g_t) S0^T q_t + sum_{j <= t} exp(u_j - g_t) (q_t . k_j) v_j ] / (max(|nq_t|, exp(-m_t)) + 1e-6)
+//   nq_t =   exp(m0 - g_t) n0 . q_t + sum_{j <= t} exp(u_j - g_t) (q_t . k_j)
+//   S    =   exp(m0 - g_last) S0 + sum_j exp(u_j - g_last) k_j v_j^T,   n likewise,   m = m_last
+// (every exponent is at most 0). A workgroup owns up to 64 value columns of one (sequence, head), a wave 16 of them; a
+// wave's part of S stays in registers in the layout that is both the accumulator of K'^T V and the B operand of Q S.
+#include "tw_common.h"
+
+struct MlstmArgs {
+  const float* proj; long ld;        // a token's row: q at q_col + h D, k at k_col + h D, v at v_col + h E,
+  int q_col, k_col, v_col;           // the gates' raw values at i_col + h and f_col + h
+  int i_col, f_col;
+  const float* i_bias; const float* f_bias;   // [H]
+  float* S; float* n; float* m;
+  const int* q_start; const int* state_slots; const int* phase;
+  int seq0;
+  float* out; long ld_out;           // [rows][H E]
+  int H, D, E, Dp, Ep;
+  float q_scale, cap;
+};
+
+__device__ __forceinline__ float ml_logsigmoid(float z) { return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z)); }
+
+__device__ __forceinline__ void ml_gates(const MlstmArgs& a, const float* row, int head, float& i_log, float& f_log) {
+  i_log = a.cap * tanhf((row[a.i_col + head] + a.i_bias[head]) / a.cap);
+  f_log = ml_logsigmoid(a.cap * tanhf((row[a.f_col + head] + a.f_bias[head]) / a.cap));
+}
+
+// grid (Ep / 16, H, n_seqs), 256 threads
+__global__ __launch_bounds__(256) void mlstm_walk_kernel(MlstmArgs a) {
+  const int seq = a.seq0 + blockIdx.z, head = blockIdx.y;
+  const int col = threadIdx.x >> 4, sl = threadIdx.x & 15;
+  const int v = blockIdx.x * 16 + col;
+  const int r0 = a.q_start[seq], r1 = a.q_start[seq + 1];
+  if (r1 <= r0) return;
+  const int slot = a.state_slots[seq], ph = a.phase[seq] & 1;
+  const int J = a.Dp / 16;
+  float* S = a.S + (((size_t)slot * a.H + head) * a.Ep + v) * a.Dp;
+  const float* n_in = a.n + (((size_t)slot * 2 + ph) * a.H + head) * a.Dp;
+  float* n_out = a.n + (((size_t)slot * 2 + (ph ^ 1)) * a.H + head) * a.Dp;
+  float s[16], nn[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    s[j] = j < J ? S[sl + 16 * j] : 0.f;
+    nn[j] = j < J ? n_in[sl + 16 * j] : 0.f;
+  }
+  float m = a.m[((size_t)slot * 2 + ph) * a.H + head];
+  for (int row_i = r0; row_i < r1; ++row_i) {
+    const float* row = a.proj + (size_t)row_i * a.ld;
+    float i_log, f_log;
+    ml_gates(a, row, head, i_log, f_log);
+    const float m_new = fmaxf(f_log + m, i_log);
+    const float keep = expf(f_log + m - m_new), take = expf(i_log - m_new);
+    m = m_new;
+    const float vv = v < a.E ? row[a.v_col + head * a.E + v] : 0.f;
+    const float* q = row + a.q_col + head * a.D;
+    const float* k = row + a.k_col + head * a.D;
+    float po = 0.f, pn = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (j < J) {
+        const int d = sl + 16 * j;
+        const float kd = d < a.D ? k[d] : 0.f, qd = d < a.D ? q[d] * a.q_scale : 0.f;
+        const float tk = take * kd;
+        s[j] = __fmaf_rn(keep, s[j], tk * vv);
+        nn[j] = __fmaf_rn(keep, nn[j], tk);
+        po = __fmaf_rn(s[j], qd, po);
+        pn = __fmaf_rn(nn[j], qd, pn);
+      }
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) {
+      po += __shfl_xor(po, o, TW_WAVE);
+      pn += __shfl_xor(pn, o, TW_WAVE);
+    }
+    if (sl == 0 && v < a.E)
+      a.out[(size_t)row_i * a.ld_out + head * a.E + v] = po / (fmaxf(fabsf(pn), expf(-m)) + 1e-6f);
+  }
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    if (j < J) S[sl + 16 * j] = s[j];
+  if (blockIdx.x == 0) {
+    if (col == 0) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        if (j < J) n_out[sl + 16 * j] = nn[j];
+    }
+    if (threadIdx.x == 0) a.m[((size_t)slot * 2 + (ph ^ 1)) * a.H + head] = m;
+  }
+}
+
+// grid (ceil(Ep / 64), H, n_seqs), 256 threads; dynamic LDS (ml_chunk_lds_floats).
+#define ML_L 16
+static size_t ml_chunk_lds_floats(int Dp) {
+  return (size_t)2 * ML_L * (Dp + 4) + (size_t)ML_L * 68 + 4 * 64 * 4 + Dp + 5 * ML_L;
+}
+
+template <int DT>      // key tiles of 16 a wave's part of S spans in registers (Dp <= 16 DT)
+__global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float ml_lds[];
+  const int seq = a.seq0 + blockIdx.z, head = blockIdx.y;
+  const int r0 = a.q_start[seq], r1 = a.q_start[seq + 1];
+  if (r1 <= r0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int Dp = a.Dp, QS = Dp + 4, tiles = Dp / 16;
+  float* Qs = ml_lds;                          // [16][Dp + 4], scaled queries
+  float* Ks = Qs + ML_L * QS;                  // [16][Dp + 4]
+  float* Vs = Ks + ML_L * QS;                  // [16][68]: this workgroup's 64 value columns
+  f32x4* part = (f32x4*)(Vs + ML_L * 68);      // [4 waves][64 lanes]
+  float* n_s = (float*)(part + 4 * 64);        // [Dp]
+  float* u_s = n_s + Dp;                       // [16] i_j - F_j (minus infinity behind the chunk's last token)
+  float* g_s = u_s + ML_L;                     // [16] running maximum, m0 included
+  float* F_s = g_s + ML_L;                     // [16]
+  float* nq_s = F_s + ML_L;                    // [16] n0 . q_t
+  const int slot = a.state_slots[seq], ph = a.phase[seq] & 1;
+  const int v0 = blockIdx.x * 64 + wave * 16;  // this wave's value columns v0 .. v0 + 15
+  const bool wave_on = v0 < a.Ep;
+  float* S = a.S + (((size_t)slot * a.H + head) * a.Ep + v0 + r) * Dp;
+  const float* n_in = a.n + (((size_t)slot * 2 + ph) * a.H + head) * Dp;
+  float* n_out = a.n + (((size_t)slot * 2 + (ph ^ 1)) * a.H + head) * Dp;
+  f32x4 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    acc[dt] = (wave_on && dt < tiles) ? *reinterpret_cast<const f32x4*>(S + dt * 16 + 4 * g) : f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int d = threadIdx.x; d < Dp; d += 256) n_s[d] = n_in[d];
+  float m0 = a.m[((size_t)slot * 2 + ph) * a.H + head];
+
+  for (int c0 = r0; c0 < r1; c0 += ML_L) {
+    const int valid = min(ML_L, r1 - c0);
+    // ---- 1: the chunk's rows and gates into LDS ------------------------------------------------------------
+    for (int i = threadIdx.x; i < ML_L * Dp; i += 256) {
+      const int t = i / Dp, d = i - t * Dp;
+      float qv = 0.f, kv = 0.f;
+      if (t < valid && d < a.D) {
+        const float* row = a.proj + (size_t)(c0 + t) * a.ld;
+        qv = row[a.q_col + head * a.D + d] * a.q_scale;
+        kv = row[a.k_col + head * a.D + d];
+      }
+      Qs[t * QS + d] = qv;
+      Ks[t * QS + d] = kv;
+    }
+    for (int i = threadIdx.x; i < ML_L * 64; i += 256) {
+      const int t = i >> 6, c = i & 63;
+      const int v = blockIdx.x * 64 + c;
+      Vs[t * 68 + c] = (t < valid && v < a.E) ? a.proj[(size_t)(c0 + t) * a.ld + a.v_col + head * a.E + v] : 0.f;
+    }
+    if (threadIdx.x < ML_L) {
+      const int t = threadIdx.x;
+      float i_log = 0.f, f_log = 0.f;
+      if (t < valid) ml_gates(a, a.proj + (size_t)(c0 + t) * a.ld, head, i_log, f_log);
+      float F = f_log;                            // inclusive running sum over the 16 lanes
+#pragma unroll
+      for (int o = 1; o < ML_L; o <<= 1) {
+        const float up = __shfl_up(F, o, TW_WAVE);
+        if (t >= o) F += up;
+      }
+      const float u = t < valid ? i_log - F : -INFINITY;
+      float best = fmaxf(u, m0);                  // running maximum, m0 included
+#pragma unroll
+      for (int o = 1; o < ML_L; o <<= 1) {
+        const float up = __shfl_up(best, o, TW_WAVE);
+        if (t >= o) best = fmaxf(best, up);
+      }
+      u_s[t] = u;
+      g_s[t] = best;
+      F_s[t] = F;
+    }
+    __syncthreads();
+    // ---- 2: K Q^T over this wave's share of the key elements; n0 . q_t ------------------------------------
+    {
+      f32x4 p = {0.f, 0.f, 0.f, 0.f};
+      for (int dt = wave; dt < tiles; dt += 4) {
+        const f32x4 kf = *reinterpret_cast<const f32x4*>(Ks + r * QS + dt * 16 + 4 * g);
+        const f32x4 qf = *reinterpret_cast<const f32x4*>(Qs + r * QS + dt * 16 + 4 * g);
+        tw_mma16(p, kf, qf);                      // p[e]: k_(4 g + e) . q_r
+      }
+      part[wave * 64 + lane] = p;
+      const int t = threadIdx.x >> 4, piece = threadIdx.x & 15;
+      float sum = 0.f;
+      for (int d = piece; d < Dp; d += 16) sum = __fmaf_rn(n_s[d], Qs[t * QS + d], sum);
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, TW_WAVE);
+      if (piece == 0) nq_s[t] = sum;
+    }
+    __syncthreads();
+    // ---- 3: weights, outputs, the new state -------------------------------------------------------------------
+    const int last = valid - 1;
+    const float g_last = g_s[last];
+    const float carry = expf(m0 - g_last);        // what is left of the state before the chunk
+    if (wave_on) {
+      f32x4 w = part[lane] + part[64 + lane] + part[128 + lane] + part[192 + lane];
+      const float g_t = g_s[r];
+      float rows = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int j = 4 * g + e;
+        w[e] = (j <= r && j < valid) ? expf(u_s[j] - g_t) * w[e] : 0.f;    // W[t = r][j]
+        rows += w[e];
+      }
+      rows = tw_rows_sum(rows);
+      const float nq = __fmaf_rn(expf(m0 - g_t), nq_s[r], rows);
+      const float den = fmaxf(fabsf(nq), expf(-(F_s[r] + g_t))) + 1e-6f;   // of token r
+      // values of keys 4 g .. 4 g + 3, column v0 + r
+      f32x4 vf;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) vf[e] = Vs[(4 * g + e) * 68 + wave * 16 + r];
+      f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        if (dt < tiles) {
+          const f32x4 qf = *reinterpret_cast<const f32x4*>(Qs + r * QS + dt * 16 + 4 * g);
+          tw_mma16_k4(o, qf, acc[dt]);            // o[e]: token 4 g + e, column v0 + r
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] *= expf(m0 - g_s[4 * g + e]);
+      tw_mma16_k4(o, w, vf);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int t = 4 * g + e;
+        const float den_t = __shfl(den, t, TW_WAVE);
+        if (t < valid && v0 + r < a.E)
+          a.out[(size_t)(c0 + t) * a.ld_out + head * a.E + v0 + r] = o[e] / den_t;
+      }
+      // S <- carry S + sum_j exp(u_j - g_last) k_j v_j^T
+      float ej[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ej[e] = (4 * g + e) < valid ? expf(u_s[4 * g + e] - g_last) : 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        if (dt < tiles) {
+          f32x4 kf;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) kf[e] = Ks[(4 * g + e) * QS + dt * 16 + r] * ej[e];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[dt][e] *= carry;
+          tw_mma16_k4(acc[dt], kf, vf);
+        }
+      }
+    }
+    for (int d = threadIdx.x; d < Dp; d += 256) {
+      float sum = carry * n_s[d];
+      for (int j = 0; j < valid; ++j) sum = __fmaf_rn(expf(u_s[j] - g_last), Ks[j * QS + d], sum);
+      n_s[d] = sum;
+    }
+    m0 = F_s[last] + g_last;
+    __syncthreads();
+  }
+  if (wave_on) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      if (dt < tiles) *reinterpret_cast<f32x4*>(S + dt * 16 + 4 * g) = acc[dt];
+  }
+  if (blockIdx.x == 0) {
+    for (int d = threadIdx.x; d < Dp; d += 256) n_out[d] = n_s[d];
+    if (threadIdx.x == 0) a.m[((size_t)slot * 2 + (ph ^ 1)) * a.H + head] = m0;
+  }
+}
+
+// Sequences seq0 .. seq0 + n_seqs - 1. walk != 0: token by token (steps of a few tokens), else in chunks of 16.
+extern "C" int tw_mlstm(const float* proj, long ld, int q_col, int k_col, int v_col, int i_col, int f_col, const float* i_bias,
+                        const float* f_bias, float* S, float* n, float* m, const int* q_start, const int* state_slots,
+                        const int* phase, int seq0, int n_seqs, float* out, long ld_out, int H, int D, int E, float q_scale,
+                        float cap, int walk, hipStream_t stream) {
+  TW_REQUIRE(proj && i_bias && f_bias && S && n && m && q_start && state_slots && phase && out);
+  TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && H > 0 && D > 0 && D <= 256 && E > 0 && cap > 0.f);
+  TW_REQUIRE(q_col >= 0 && k_col >= 0 && v_col >= 0 && i_col >= 0 && f_col >= 0);
+  TW_REQUIRE(ld >= q_col + (long)H * D && ld >= k_col + (long)H * D && ld >= v_col + (long)H * E && ld >= i_col + (long)H &&
+             ld >= f_col + (long)H && ld_out >= (long)H * E);
+  if (n_seqs == 0) return 0;
+  const int Dp = (D + 15) / 16 * 16, Ep = (E + 15) / 16 * 16;
+  TW_REQUIRE((uintptr_t)S % 16 == 0);
+  MlstmArgs a{proj, ld, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, S, n, m, q_start, state_slots, phase, seq0,
+              out, ld_out, H, D, E, Dp, Ep, q_scale, cap};
+  if (walk) {
+    mlstm_walk_kernel<<<dim3(Ep / 16, H, n_seqs), 256, 0, stream>>>(a);
+    return TW_LAUNCH_RESULT();
+  }
+  const dim3 grid(tw_div_up(Ep, 64), H, n_seqs);
+  const size_t lds = ml_chunk_lds_floats(Dp) * sizeof(float);
+  if (Dp <= 64) mlstm_chunk_kernel<4><<<grid, 256, lds, stream>>>(a);
+  else if (Dp <= 128) mlstm_chunk_kernel<8><<<grid, 256, lds, stream>>>(a);
+  else mlstm_chunk_kernel<16><<<grid, 256, lds, stream>>>(a);
+  return TW_LAUNCH_RESULT();
+}

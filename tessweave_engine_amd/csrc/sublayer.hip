@@ -173,3 +173,183 @@ extern "C" int tw_relu_squared(int dtype, void* x, long ld, int n, int cols, con
   else return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
 }
+
+// ---- a norm on the sublayer's RESULT: x <- x + mult * w * unit(y) -------------------------------------------------
+// y is a sublayer's float32 result (or split-K partial sums that are added up here, in index order); its statistic is
+// float32; the sum goes back into the float32 stream x and, rounded once, to `out` in the compute type, which is what
+// the next sublayer's products read (such an arrangement's sublayers read the stream itself). A block a row, four
+// elements a thread and pass where rows and addresses allow; the row of y stays in registers between the two passes
+// up to 4,096 elements, longer rows are read again.
+struct AddNormedArgs {
+  float* x;
+  const float* y; long ldy;
+  const float* add; int splits; size_t add_stride;
+  const float* w;
+  void* out;
+  int hidden;
+  float mult, eps;
+};
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void add_normed_kernel(AddNormedArgs a) {
+  __shared__ float lds[16];
+  constexpr int W = VEC ? 4 : 1;
+  constexpr int KEEP = 4;
+  const int row = blockIdx.x;
+  const int units = a.hidden / W;
+  float* x = a.x + (size_t)row * a.hidden;
+  auto load = [&](int u, float* v) {
+#pragma unroll
+    for (int e = 0; e < W; ++e) v[e] = 0.f;
+    if (a.add) {
+      for (int s = 0; s < a.splits; ++s) {
+        const float* p = a.add + s * a.add_stride + (size_t)row * a.hidden + (size_t)u * W;
+        if (VEC) {
+          const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+          for (int e = 0; e < W; ++e) v[e] += t[e];
+        } else {
+          v[0] += p[0];
+        }
+      }
+    } else {
+      const float* p = a.y + (size_t)row * a.ldy + (size_t)u * W;
+      if (VEC) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+        for (int e = 0; e < W; ++e) v[e] = t[e];
+      } else {
+        v[0] = p[0];
+      }
+    }
+  };
+  float kept[KEEP][W];
+  float ss = 0.f;
+  int i = 0;
+  for (int u = threadIdx.x; u < units; u += blockDim.x, ++i) {
+    float v[W];
+    load(u, v);
+#pragma unroll
+    for (int e = 0; e < W; ++e) ss = __fmaf_rn(v[e], v[e], ss);
+    if (i < KEEP) {
+#pragma unroll
+      for (int e = 0; e < W; ++e) kept[i][e] = v[e];
+    }
+  }
+  const float total = tw_block_sum(ss, lds);
+  const float f = a.mult / sqrtf(total / (float)a.hidden + a.eps);
+  T* out = a.out ? (T*)a.out + (size_t)row * a.hidden : nullptr;
+  i = 0;
+  for (int u = threadIdx.x; u < units; u += blockDim.x, ++i) {
+    float v[W];
+    if (i < KEEP) {
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] = kept[i][e];
+    } else {
+      load(u, v);
+    }
+#pragma unroll
+    for (int e = 0; e < W; ++e) {
+      const int c = u * W + e;
+      const float r = __fmaf_rn(v[e] * f, a.w[c], x[c]);
+      x[c] = r;
+      if (out) out[c] = tw_from_float<T>(r);
+    }
+  }
+}
+
+extern "C" int tw_add_normed(int out_dtype, float* x, const float* y, long ldy, const float* add, int splits, long add_stride,
+                             const float* w, void* out, int n, int hidden, float mult, float eps, hipStream_t stream) {
+  TW_REQUIRE(x && w && (y || add) && n >= 0 && hidden > 0 && eps > 0.f);
+  TW_REQUIRE(add == nullptr || (splits > 0 && add_stride >= (long)n * hidden));
+  TW_REQUIRE(add != nullptr || ldy >= hidden);
+  if (n == 0) return 0;
+  AddNormedArgs a{x, add ? nullptr : y, ldy, add, splits, (size_t)add_stride, w, out, hidden, mult, eps};
+  const bool vec = hidden % 4 == 0 && (add ? ((uintptr_t)add % 16 == 0 && add_stride % 4 == 0)
+                                           : ((uintptr_t)y % 16 == 0 && ldy % 4 == 0));
+  if (out_dtype == TW_DTYPE_BF16) {
+    if (vec) add_normed_kernel<bf16_t, true><<<n, 256, 0, stream>>>(a);
+    else add_normed_kernel<bf16_t, false><<<n, 256, 0, stream>>>(a);
+  } else if (out_dtype == TW_DTYPE_F32) {
+    if (vec) add_normed_kernel<float, true><<<n, 256, 0, stream>>>(a);
+    else add_normed_kernel<float, false><<<n, 256, 0, stream>>>(a);
+  } else {
+    return TW_ERR_BAD_ARGUMENT;
+  }
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- activations of a plain product, in place: kind 1 max(x, 0)^2 (above), 2 the exact gelu, x Phi(x) -------------
+__device__ __forceinline__ float sl_act(float v, int kind) {
+  if (kind == 2) return 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
+  v = fmaxf(v, 0.f);
+  return v * v;
+}
+
+template <typename T>
+__global__ void activation_kernel(T* __restrict__ x, long ld, int cols, long total, const float* __restrict__ partial, int splits,
+                                  int kind) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  T* p = x + (i / cols) * ld + i % cols;
+  float v = 0.f;
+  if (partial) {
+    for (int s = 0; s < splits; ++s) v += partial[(size_t)s * total + i];
+  } else {
+    v = tw_to_float(*p);
+  }
+  *p = tw_from_float<T>(sl_act(v, kind));
+}
+
+extern "C" int tw_activation(int dtype, void* x, long ld, int n, int cols, const float* partial, int splits, int kind,
+                             hipStream_t stream) {
+  TW_REQUIRE(x && n >= 0 && cols > 0 && ld >= cols && (partial == nullptr || splits > 0) && (kind == 1 || kind == 2));
+  if (n == 0) return 0;
+  const long total = (long)n * cols;
+  const int blocks = tw_div_up(total, 256);
+  if (dtype == TW_DTYPE_BF16) activation_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, ld, cols, total, partial, splits, kind);
+  else if (dtype == TW_DTYPE_F32) activation_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, ld, cols, total, partial, splits, kind);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- out <- out * sigmoid(gate), element by element (an output gate in front of the output product) ---------------
+template <typename T, typename G>
+__global__ void sigmoid_gate_kernel(T* __restrict__ out, long ld_out, const G* __restrict__ gate, long ld_g, int cols, long total) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long row = i / cols;
+  const int col = (int)(i % cols);
+  T* p = out + row * ld_out + col;
+  const float z = tw_to_float(gate[row * ld_g + col]);
+  *p = tw_from_float<T>(tw_to_float(*p) / (1.f + expf(-z)));
+}
+
+extern "C" int tw_sigmoid_gate(int dtype, void* out, long ld_out, const void* gate, long ld_g, int gate_f32, int n, int cols,
+                               hipStream_t stream) {
+  TW_REQUIRE(out && gate && n >= 0 && cols > 0 && ld_out >= cols && ld_g >= cols);
+  if (n == 0) return 0;
+  const long total = (long)n * cols;
+  const int blocks = tw_div_up(total, 256);
+  if (dtype == TW_DTYPE_BF16 && gate_f32)
+    sigmoid_gate_kernel<bf16_t, float><<<blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const float*)gate, ld_g, cols, total);
+  else if (dtype == TW_DTYPE_BF16)
+    sigmoid_gate_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)gate, ld_g, cols, total);
+  else if (dtype == TW_DTYPE_F32)
+    sigmoid_gate_kernel<float, float><<<blocks, 256, 0, stream>>>((float*)out, ld_out, (const float*)gate, ld_g, cols, total);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- x <- cap * tanh(x / cap) over float32 values (a soft cap of the logits) ---------------------------------------
+__global__ void softcap_values_kernel(float* __restrict__ x, long total, float cap) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" int tw_softcap_values(float* x, long total, float cap, hipStream_t stream) {
+  TW_REQUIRE(x && total >= 0 && cap > 0.f);
+  if (total == 0) return 0;
+  softcap_values_kernel<<<tw_div_up(total, 256), 256, 0, stream>>>(x, total, cap);
+  return TW_LAUNCH_RESULT();
+}

@@ -49,7 +49,7 @@ _SIGNATURES = {
     "tw_attn_mixed_splits": (I, [I, I]),
     "tw_attn_mixed_prefill_splits": (I, [I, I, I]),
     "tw_attn_mixed_workspace_floats": (L, [I, I, I, I, I]),
-    "tw_attn_mixed": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P]),
+    "tw_attn_mixed": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, P, P, P, L, I, I, I, I, I, I, I, F, F, I, P]),
     "tw_kv_store": (I, [I, P, L, I, I, P, P, P, I, I, I, I, I, P]),
     "tw_residual_norm": (I, [I, P, P, L, P, I, L, P, P, P, I, I, F, F, P]),
     "tw_relu_squared": (I, [I, P, L, I, I, P, I, P]),
@@ -57,7 +57,7 @@ _SIGNATURES = {
     "tw_latent_finish": (I, [I, P, L, I, I, I, P, P, P, P, L, P, L, I, I, I, I, P, P, P, I, I, I, I, I, I, I, F, P]),
     "tw_latent_decode_splits": (I, [I, I, I]),
     "tw_latent_decode_workspace_floats": (L, [I, I, I, I]),
-    "tw_latent_decode": (I, [I, P, L, P, P, P, I, P, P, I, P, L, P, L, I, I, I, I, F, I, P]),
+    "tw_latent_decode": (I, [I, P, L, P, P, P, I, P, P, I, P, L, P, L, I, I, I, I, F, I, P, P]),
     "tw_latent_gather": (I, [I, P, P, I, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_latent_expand_store": (I, [I, P, L, P, I, I, P, P, I, I, I, I, I, I, I, P]),
     "tw_head_linear": (I, [I, P, L, I, P, P, L, I, I, I, I, I, P]),
@@ -68,10 +68,16 @@ _SIGNATURES = {
     "tw_rmsnorm_pair": (I, [I, P, P, P, P, P, I, I, F, P]),
     "tw_scale_values": (I, [P, L, F, P]),
     "tw_delta_rule": (I, [P, L, I, I, I, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, F, P]),
-    "tw_head_norm_gate": (I, [I, P, L, P, L, P, P, L, I, I, I, F, P]),
-    "tw_moe_route": (I, [I, P, L, P, I, I, I, I, P, P, P]),
+    "tw_head_norm_gate": (I, [I, P, L, P, L, P, P, L, I, I, I, F, I, I, P]),
+    "tw_moe_route": (I, [I, P, L, P, P, I, I, I, I, I, P, P, P]),
     "tw_moe_capacity": (L, [L, I]),
-    "tw_moe_experts": (I, [I, P, L, P, P, I, I, I, P, P, P, I, I, I, F, P, P, P, P, P, P, I, P, L, P]),
+    "tw_moe_experts": (I, [I, P, L, P, P, I, I, I, P, P, P, I, I, I, F, P, P, P, P, P, P, I, P, L, I, I, P]),
+    "tw_add_normed": (I, [I, P, P, L, P, I, L, P, P, I, I, F, F, P]),
+    "tw_activation": (I, [I, P, L, I, I, P, I, I, P]),
+    "tw_sigmoid_gate": (I, [I, P, L, P, L, I, I, I, P]),
+    "tw_softcap_values": (I, [P, L, F, P]),
+    "tw_qk_finish": (I, [I, P, L, I, I, P, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, I, F, P]),
+    "tw_mlstm": (I, [P, L, I, I, I, I, I, P, P, P, P, P, P, P, P, I, I, P, L, I, I, I, F, F, I, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),
     "tw_sample_rows": (I, [P, L, I, I, P, P, P, P, P, L, P]),

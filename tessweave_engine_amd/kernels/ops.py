@@ -340,7 +340,7 @@ def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_
     return out
 
 
-LINEAR_ACTIVATIONS = {"relu_squared": 1}
+LINEAR_ACTIVATIONS = {"relu_squared": 1, "gelu": 2}
 
 
 def can_linear_act(x, weight):
@@ -709,13 +709,14 @@ def kv_store(src, k_col, v_col, slots, keys, values, kv_heads, key_dim, value_di
 
 
 def attn_mixed(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_q_len, out, q_heads, kv_heads, scale,
-               window=0, talk=None, sink=None, slopes=None, out_scale=1.0, splits=1, workspace=None):
+               window=0, talk=None, sink=None, slopes=None, out_scale=1.0, splits=1, workspace=None, keep_first=0):
     """Attention of sequences seq0 .. seq0 + n_seqs - 1 whose scores are mixed across heads before the softmax.
 
     q [rows, >= q_heads * key_dim] (head h at columns h * key_dim), keys [pages, kv_heads, page, key_dim], values
     [pages, kv_heads, value_dim, page], out [rows, q_heads * value_dim]. talk float32 [H, H] mixes the scores
     (None: no mixing), slopes float32 [H] take slope * distance off the raw scores, sink float32 [H] adds exp(sink)
-    to the softmax's denominator. splits > 1 cuts every tile's keys into ranges; needs a workspace
+    to the softmax's denominator. keep_first: with a window, the sequence's first keep_first keys stay visible to every later
+    query (at their true positions). splits > 1 cuts every tile's keys into ranges; needs a workspace
     (`attn_mixed_workspace_floats`).
     """
     key_dim, value_dim, page = keys.shape[3], values.shape[2], keys.shape[2]
@@ -741,7 +742,7 @@ def attn_mixed(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_
                                   int(n_seqs), int(max_q_len), _dev(out), ldo,
                                   _dev(talk) if talk is not None else None, _dev(sink) if sink is not None else None,
                                   _dev(slopes) if slopes is not None else None, ws_ptr, ws_floats, q_heads, kv_heads,
-                                  key_dim, value_dim, page, int(window or 0), float(scale), float(out_scale), int(splits),
+                                  key_dim, value_dim, page, int(window or 0), int(keep_first or 0), float(scale), float(out_scale), int(splits),
                                   _stream()), "attn_mixed")
     return out
 
@@ -870,12 +871,14 @@ def latent_decode_workspace_floats(n_seqs, heads, latent_dev, splits):
     return int(library().tw_latent_decode_workspace_floats(int(n_seqs), int(heads), int(latent_dev), int(splits)))
 
 
-def latent_decode(q, keys, values, block_table, q_start, kv_len, n_seqs, out, heads, scale, splits=1, workspace=None):
+def latent_decode(q, keys, values, block_table, q_start, kv_len, n_seqs, out, heads, scale, splits=1, workspace=None, sink=None):
     """Attention of sequences 0 .. n_seqs - 1, ONE query token each, all heads against the one cached head: softmax of
     scale * q_a . key over the sequence's keys, times the values (the first latent_dev elements of the key rows).
     q [rows, heads * K] (head a at a * K), keys [pages, 1, page, K], values [pages, 1, latent_dev, page] (the same
     elements, transposed inside a page), out [rows, heads * latent_dev]. splits > 1 cuts every sequence's keys into
-    ranges for separate workgroups; needs a float32 workspace of `latent_decode_workspace_floats` floats."""
+    ranges for separate workgroups; needs a float32 workspace of `latent_decode_workspace_floats` floats. sink float32
+    [heads]: exp(sink_a) more in head a's denominator (no key, no value, not scaled)."""
+    _need(sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == heads), "sink must be float32 [heads]")
     page, K = keys.shape[2], keys.shape[3]
     Lp = values.shape[2]
     nq, wq, ldq = _rows(q, "q")
@@ -895,7 +898,7 @@ def latent_decode(q, keys, values, block_table, q_start, kv_len, n_seqs, out, he
                                      _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
                                      _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"), int(n_seqs),
                                      _dev(out), ldo, ws_ptr, ws_floats, int(heads), K, Lp, page, float(scale), int(splits),
-                                     _stream()), "latent_decode")
+                                     _dev(sink) if sink is not None else None, _stream()), "latent_decode")
     return out
 
 
@@ -1083,32 +1086,44 @@ def delta_rule(qkv, q_col, k_col, v_col, ab, b_col, a_col, A_log, dt_bias, state
     return out
 
 
-def head_norm_gate(o, gate, weight, out, heads, value_dim, eps):
-    """out[n, h, e] = o[n, h, e] / sqrt(mean_e o^2 + eps) * weight[e] * silu(gate[n, h, e]); o and gate float32, weight
-    float32 [value_dim] shared by the heads, out of the compute type."""
+def head_norm_gate(o, gate, weight, out, heads, value_dim, eps, gate_activation="silu"):
+    """out[n, h, e] = o[n, h, e] / sqrt(mean_e o^2 + eps) * weight[e] * act(gate[n, h, e]); o and gate float32, weight
+    float32 [value_dim] shared by the heads or [heads * value_dim] with one vector a head, out of the compute type;
+    act the SiLU or ("sigmoid") the sigmoid of the gate."""
+    _need(gate_activation in ("silu", "sigmoid"), "the gate passes 'silu' or 'sigmoid'")
     n, wo, ld_o = _rows(o, "o")
     ng, wg, ld_g = _rows(gate, "gate")
     nn, wn, ld_n = _rows(out, "out")
     _need(o.dtype == torch.float32 and gate.dtype == torch.float32, "o and gate are float32")
-    _need(ng == n and nn == n and min(wo, wg, wn) >= heads * value_dim and weight.numel() == value_dim, "head_norm_gate shapes do not agree")
+    _need(ng == n and nn == n and min(wo, wg, wn) >= heads * value_dim and weight.numel() in (value_dim, heads * value_dim)
+          and weight.is_contiguous(), "head_norm_gate shapes do not agree")
+    per_head = 1 if (weight.numel() == heads * value_dim and heads > 1) else 0
     check(library().tw_head_norm_gate(dtype_id(out.dtype), _dev(o), ld_o, _dev(gate), ld_g, _dev(weight, torch.float32, "weight"),
-                                      _dev(out), ld_n, n, int(heads), int(value_dim), float(eps), _stream()), "head_norm_gate")
+                                      _dev(out), ld_n, n, int(heads), int(value_dim), float(eps), per_head,
+                                      1 if gate_activation == "sigmoid" else 0, _stream()), "head_norm_gate")
     return out
 
 
 MOE_MAX_EXPERTS = 1024
 
 
-def moe_route(h, router, top, ids, weights):
-    """ids[n, top], weights[n, top]: per row of h the `top` experts with the largest router logits router @ h (float32
-    products of h's values as they are; the lowest index wins a tie), and the sigmoid of each chosen logit."""
+MOE_WEIGHTS = {"sigmoid": 0, "softmax_chosen": 1}
+
+
+def moe_route(h, router, top, ids, weights, bias=None, weighting="sigmoid"):
+    """ids[n, top], weights[n, top]: per row of h the `top` experts with the largest router logits router @ h + bias
+    (float32 products of h's values as they are; the lowest index wins a tie), and per chosen logit its sigmoid or
+    ("softmax_chosen") its share of the softmax over the chosen logits alone."""
+    _need(weighting in MOE_WEIGHTS, "a router's weights are 'sigmoid' or 'softmax_chosen'")
     n, C, ld_h = _rows(h, "h")
     X = router.shape[0]
     _need(router.dtype == torch.float32 and router.is_contiguous() and tuple(router.shape) == (X, C), "the router is float32 [experts, C]")
     _need(0 < top <= X <= MOE_MAX_EXPERTS, f"1 to {MOE_MAX_EXPERTS} experts, of which at most all are chosen")
     _need(ids.is_contiguous() and weights.is_contiguous() and tuple(ids.shape) == (n, top) and tuple(weights.shape) == (n, top),
           "ids and weights are [n, top]")
-    check(library().tw_moe_route(dtype_id(h.dtype), _dev(h), ld_h, _dev(router), n, C, X, int(top), _dev(ids, torch.int32, "ids"),
+    _need(bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == X), "the router's bias is float32 [experts]")
+    check(library().tw_moe_route(dtype_id(h.dtype), _dev(h), ld_h, _dev(router), _dev(bias) if bias is not None else None,
+                                 MOE_WEIGHTS[weighting], n, C, X, int(top), _dev(ids, torch.int32, "ids"),
                                  _dev(weights, torch.float32, "weights"), _stream()), "moe_route")
     return ids, weights
 
@@ -1136,14 +1151,20 @@ def moe_blocked(w):
     return w.reshape(X, N16 // 16, 16, K // (4 * epf), 4, epf).permute(0, 1, 3, 4, 2, 5).contiguous().reshape(X, N16, K)
 
 
-def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch):
-    """x[n] += sum over a row's chosen experts e of down_e(glu(gate_e y, up_e y)), y = round(weights * h[n]), glu the
+MOE_KINDS = {"swish_limited": 0, "gelu": 1}
+
+
+def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch, kind="swish_limited", accumulate=True):
+    """kind "gelu" (gate None): x[n] (+)= sum over a row's chosen experts e of weights_e * down_e(gelu(up_e h[n])), the exact
+    gelu; accumulate=False writes x instead of adding to it. kind "swish_limited": x[n] += sum over a row's chosen experts e of down_e(glu(gate_e y, up_e y)), y = round(weights * h[n]), glu the
     limited swish with LIMIT. gate, up [X, Fd, Cd], down [X, C16, Fd] in h's type, zero padded (Fd, Cd: `moe_pad` of the
     sizes, C16: C rounded up to 16) and laid out by `moe_blocked`. scratch(tag, shape, dtype) hands out the step's scratch tensors."""
     n, C, ld_h = _rows(h, "h")
     top = ids.shape[1]
-    X, Fd, Cd = gate.shape
-    _need(gate.is_contiguous() and up.is_contiguous() and down.is_contiguous() and gate.dtype == up.dtype == down.dtype == h.dtype,
+    _need(kind in MOE_KINDS and (gate is None) == (kind == "gelu"), "experts are 'swish_limited' (with a gate) or 'gelu' (without)")
+    X, Fd, Cd = up.shape
+    _need((gate is None or (gate.is_contiguous() and gate.dtype == h.dtype and tuple(gate.shape) == (X, Fd, Cd)))
+          and up.is_contiguous() and down.is_contiguous() and up.dtype == down.dtype == h.dtype,
           "the experts' matrices are contiguous and of h's type")
     _need(tuple(up.shape) == (X, Fd, Cd) and tuple(down.shape) == (X, (C + 15) // 16 * 16, Fd) and Cd == moe_pad(C) and Fd % 32 == 0,
           "the experts' matrices are [X, Fd, Cd] and [X, C16, Fd]")
@@ -1159,7 +1180,131 @@ def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch):
     act = scratch("moe.act", (capacity, Fd), h.dtype)
     ys = scratch("moe.ys", (capacity, C), torch.float32)
     check(library().tw_moe_experts(dtype_id(h.dtype), _dev(h), ld_h, _dev(ids, torch.int32, "ids"),
-                                   _dev(weights, torch.float32, "weights"), n, top, X, _dev(gate), _dev(up), _dev(down), C, Cd, Fd,
+                                   _dev(weights, torch.float32, "weights"), n, top, X, _dev(gate) if gate is not None else None,
+                                   _dev(up), _dev(down), C, Cd, Fd,
                                    float(limit), _dev(pos), _dev(src_item), _dev(tile_expert), _dev(xs), _dev(act), _dev(ys),
-                                   capacity, _dev(x), ld_x, _stream()), "moe_experts")
+                                   capacity, _dev(x), ld_x, MOE_KINDS[kind], 1 if accumulate else 0, _stream()), "moe_experts")
     return x
+
+
+# ---- a norm on a sublayer's result, output gates, convolved and normed queries and keys, the mLSTM ------------------------
+
+def add_normed(x, weight, eps, mult=1.0, y=None, add=None, out=None):
+    """x <- x + mult * weight * unit(y), unit(v) = v / sqrt(mean(v^2) + eps); x float32 [n, hidden] in place.
+
+    y: float32 [n, hidden] (rows may be strided), or add: float32 [splits, n, hidden] partial sums added up here;
+    out: the new x once more, rounded to its type (the compute type)."""
+    _need(x.dim() == 2 and x.is_contiguous() and x.dtype == torch.float32, "add_normed: x must be contiguous float32 [n, hidden]")
+    n, hidden = x.shape
+    _need(weight.numel() == hidden and weight.dtype == torch.float32 and weight.is_contiguous(), "the norm weight must be float32 [hidden]")
+    _need((y is None) != (add is None), "either y or partial sums")
+    ldy, splits, stride = 0, 0, 0
+    if y is not None:
+        ny, cy, ldy = _rows(y, "y")
+        _need((ny, cy) == (n, hidden) and y.dtype == torch.float32, "y must be float32 [n, hidden]")
+    else:
+        _need(add.dim() == 3 and add.is_contiguous() and tuple(add.shape[1:]) == (n, hidden) and add.dtype == torch.float32,
+              "partial sums must be float32 [splits, n, hidden]")
+        splits, stride = add.shape[0], n * hidden
+    out_dtype = F32
+    if out is not None:
+        _need(out.is_contiguous() and tuple(out.shape) == (n, hidden), "out must be contiguous [n, hidden]")
+        out_dtype = dtype_id(out.dtype)
+    check(library().tw_add_normed(out_dtype, _dev(x), _dev(y) if y is not None else None, ldy,
+                                  _dev(add) if add is not None else None, splits, stride, _dev(weight),
+                                  _dev(out) if out is not None else None, n, hidden, float(mult), float(eps), _stream()),
+          "add_normed")
+    return x
+
+
+def activation(x, kind, partial=None):
+    """x <- act(x) in place (rows may be strided), act "relu_squared" or "gelu" (the exact one); with PARTIAL (float32
+    [splits, n, cols], split-K sums of the product before) x <- act(sum of the splits) instead, rounded once."""
+    _need(kind in LINEAR_ACTIVATIONS, "an activation is 'relu_squared' or 'gelu'")
+    n, cols, ld = _rows(x, "x")
+    splits = 0
+    if partial is not None:
+        _need(partial.dim() == 3 and partial.is_contiguous() and tuple(partial.shape[1:]) == (n, cols)
+              and partial.dtype == torch.float32, "partial sums must be float32 [splits, n, cols]")
+        splits = partial.shape[0]
+    check(library().tw_activation(dtype_id(x.dtype), _dev(x), ld, n, cols, _dev(partial) if partial is not None else None,
+                                  splits, LINEAR_ACTIVATIONS[kind], _stream()), "activation")
+    return x
+
+
+def sigmoid_gate(out, gate):
+    """out <- out * sigmoid(gate), element by element; gate float32 or of out's type, rows of both may be strided."""
+    n, cols, ld_out = _rows(out, "out")
+    ng, cg, ld_g = _rows(gate, "gate")
+    _need((ng, cg) == (n, cols) and gate.dtype in (torch.float32, out.dtype), "gate must be [n, cols], float32 or of out's type")
+    check(library().tw_sigmoid_gate(dtype_id(out.dtype), _dev(out), ld_out, _dev(gate), ld_g,
+                                    1 if gate.dtype == torch.float32 else 0, n, cols, _stream()), "sigmoid_gate")
+    return out
+
+
+def softcap_values(x, cap):
+    """x <- cap * tanh(x / cap) over a contiguous float32 tensor, in place."""
+    _need(x.dtype == torch.float32 and x.is_contiguous() and float(cap) > 0, "softcap_values takes contiguous float32 and a positive cap")
+    check(library().tw_softcap_values(_dev(x), x.numel(), float(cap), _stream()), "softcap_values")
+    return x
+
+
+def qk_finish(src, q_col, k_col, q_weight, k_weight, cos, sin, q_out, keys, values, slots, q_heads, kv_heads, dim, rot,
+              eps, adjacent=False):
+    """Per token: q <- rotate(q_weight * unit(q)), k <- rotate(k_weight * unit(k)), v = k as it came; unit over the WHOLE
+    row of q (q_heads * dim elements at src[:, q_col:]) and of k (kv_heads * dim at k_col), rotation of the first `rot`
+    elements of every head. src float32. q_out [n, q_heads * dim_dev] in the compute type (tails of zeros); keys
+    [pages, kv_heads, page, dim_dev], values [pages, kv_heads, dim_dev, page]; slots[n] the token's page slot (-1: not stored)."""
+    n, width, ld = _rows(src, "src")
+    nq, wq, ld_q = _rows(q_out, "q_out")
+    page, dim_dev = keys.shape[2], keys.shape[3]
+    _need(src.dtype == torch.float32 and nq == n and wq == q_heads * dim_dev, "qk_finish: src float32, q_out [n, q_heads * dim_dev]")
+    _need(keys.is_contiguous() and values.is_contiguous() and keys.dtype == values.dtype == q_out.dtype
+          and tuple(keys.shape[1:]) == (kv_heads, page, dim_dev) and tuple(values.shape) == (keys.shape[0], kv_heads, dim_dev, page),
+          "keys [pages, kv_heads, page, dim_dev], values [pages, kv_heads, dim_dev, page] of q_out's type")
+    _need(q_weight.dtype == torch.float32 and q_weight.is_contiguous() and q_weight.numel() == q_heads * dim
+          and k_weight.dtype == torch.float32 and k_weight.is_contiguous() and k_weight.numel() == kv_heads * dim,
+          "the norms' weights are float32 over the whole rows")
+    _need(q_col + q_heads * dim <= width and k_col + kv_heads * dim <= width and slots.numel() == n and dim <= dim_dev,
+          "qk_finish: columns exceed the rows, or not one slot per row")
+    if rot:
+        _need(cos is not None and cos.dtype == torch.float32 and cos.is_contiguous() and tuple(cos.shape) == (n, rot // 2)
+              and tuple(sin.shape) == (n, rot // 2), "cos and sin are float32 [n, rot / 2]")
+    check(library().tw_qk_finish(dtype_id(q_out.dtype), _dev(src), ld, int(q_col), int(k_col), _dev(q_weight), _dev(k_weight),
+                                 _dev(cos) if rot else None, _dev(sin) if rot else None, _dev(q_out), ld_q, _dev(keys),
+                                 _dev(values), _dev(slots, torch.int32, "slots"), n, int(q_heads), int(kv_heads), int(dim),
+                                 dim_dev, int(rot), 1 if adjacent else 0, page, float(eps), _stream()), "qk_finish")
+    return q_out
+
+
+MLSTM_WALK_TOKENS = 4          # sequences with up to this many tokens in a step are walked token by token
+
+
+def mlstm(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, S, n_state, m_state, q_start, state_slots, phase, seq0,
+          n_seqs, out, heads, dim, value_dim, q_scale, cap, walk):
+    """The mLSTM's matrix memory over sequences seq0 .. seq0 + n_seqs - 1 of a step. proj float32 rows with q, k
+    (heads * dim each), v (heads * value_dim) and the two gates' raw values (heads each) at the given columns; i_bias,
+    f_bias float32 [heads]. S float32 [requests, heads, value_dev, dim_dev], n_state [requests, 2, heads, dim_dev], m_state
+    [requests, 2, heads] (copy phase[s] is read, the other written). out float32 [rows, heads * value_dim]: S^T q over its
+    denominator. walk: token by token (steps of a few tokens a sequence), else chunks of 16 on the matrix unit."""
+    n, width, ld = _rows(proj, "proj")
+    no, wo, ld_out = _rows(out, "out")
+    dim_dev, value_dev = (dim + 15) // 16 * 16, (value_dim + 15) // 16 * 16
+    _need(proj.dtype == torch.float32 and out.dtype == torch.float32 and no == n and wo == heads * value_dim, "mlstm: float32 rows")
+    _need(1 <= dim <= 256, "the mLSTM kernels take key sizes up to 256")
+    _need(max(q_col, k_col) + heads * dim <= width and v_col + heads * value_dim <= width and max(i_col, f_col) + heads <= width,
+          "mlstm: columns exceed the rows")
+    requests = S.shape[0]
+    for t, shape, name in ((S, (requests, heads, value_dev, dim_dev), "S"), (n_state, (requests, 2, heads, dim_dev), "n"),
+                           (m_state, (requests, 2, heads), "m")):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == shape, f"mlstm: state {name} must be float32 {shape}")
+    for t, name in ((i_bias, "i_bias"), (f_bias, "f_bias")):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == heads, f"{name} must be float32 [heads]")
+    _need(q_start.numel() >= seq0 + n_seqs + 1 and state_slots.numel() >= seq0 + n_seqs and phase.numel() >= seq0 + n_seqs,
+          "sequence metadata is too short")
+    check(library().tw_mlstm(_dev(proj), ld, int(q_col), int(k_col), int(v_col), int(i_col), int(f_col), _dev(i_bias), _dev(f_bias),
+                             _dev(S), _dev(n_state), _dev(m_state), _dev(q_start, torch.int32, "q_start"),
+                             _dev(state_slots, torch.int32, "state_slots"), _dev(phase, torch.int32, "phase"), int(seq0),
+                             int(n_seqs), _dev(out), ld_out, int(heads), int(dim), int(value_dim), float(q_scale), float(cap),
+                             1 if walk else 0, _stream()), "mlstm")
+    return out

@@ -4,8 +4,8 @@ from .linear import JoinedLinear, Linear
 from .norms import RMSNorm
 from .positions import NoPositionEncoding, RotaryEmbedding
 from .attention import GroupedQueryAttention
-from .feedforward import GatedFeedForward, ReluSquaredFeedForward, SwiGLU
-from .blocks import DepthMixedBlock, ParallelBlock, PostNormBlock, PreNormBlock
+from .feedforward import GatedFeedForward, PlainFeedForward, ReluSquaredFeedForward, SwiGLU
+from .blocks import DepthMixedBlock, ParallelBlock, PostNormBlock, PreNormBlock, ResultNormBlock
 from .embedding import HashedPairEmbedding, OutputHead, PositionedEmbedding, TokenEmbedding
 from .convolution import CausalConv
 from .parallel import GatedLinearRecurrence, MixedHeadAttention, MixerBranch, ParallelMixer
@@ -14,6 +14,8 @@ from .latent import LatentAttention
 from .retention import Retention
 from .delta import GatedDeltaRule
 from .experts import RoutedExperts
+from .mlstm import MatrixLSTM
+from .windowed import ConvolvedWindowAttention
 from .model import DecoderModel, walk
 
 __all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer", "Norm", "Part", "PositionEncoding",
@@ -23,4 +25,5 @@ __all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer",
            "GatedLinearRecurrence", "MixedHeadAttention", "MixerBranch", "ParallelMixer", "SideTable", "TokenSideInput",
            "HashedPairEmbedding", "LatentAttention", "PostNormBlock", "ReluSquaredFeedForward", "Retention",
            "GatedDeltaRule", "ParallelBlock", "RoutedExperts",
+           "ConvolvedWindowAttention", "MatrixLSTM", "PlainFeedForward", "ResultNormBlock",
            "DecoderModel", "walk"]

@@ -155,6 +155,62 @@ class PostNormBlock(Block):
         return None
 
 
+class ResultNormBlock(Block):
+    """A norm on each sublayer's RESULT, scaled into the stream:
+
+        x <- x + mult * norm1(mixer(x));  x <- x + mult * norm2(ff(x))
+
+    The sublayers read the stream x itself (rounded to the compute type). mixer_norm, ffn_norm: `RMSNorm` parts (weight
+    and eps; norm, scaling, sum and the rounding for the next sublayer are one kernel, which also adds up split-K
+    partial sums a sublayer leaves pending). ffn / ffn_norm may be None: the layer then has only the first sublayer.
+    The mixer and the feed-forward must take `accumulate=False` (their result alone, not added into the stream)."""
+
+    def __init__(self, hidden, mixer, mixer_norm, ffn=None, ffn_norm=None, mult=1.0, unused_names=()):
+        """unused_names: tensors a checkpoint may hold for this layer that nothing reads (the norm of a feed-forward the
+        layer does not have): accepted if present, never required."""
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.hidden, self.mult = int(hidden), float(mult)
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = mixer, mixer_norm, ffn, ffn_norm
+        self.unused_names = tuple(unused_names)
+
+    def parts(self):
+        return [p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None]
+
+    def tensor_specs(self):
+        specs = [s for p in self.parts() for s in p.tensor_specs()]
+        return specs + [TensorSpec(name, (1,), VECTOR, optional_alias_of="(unused)") for name in self.unused_names]
+
+    def bind(self, tensors, dtype, device):
+        for p in self.parts():
+            p.bind(tensors, dtype, device)
+
+    def _rounded(self, ctx, x):
+        """The stream in the compute type: what the part before left, else rounded now (float32 runs read x itself)."""
+        h = ctx.shared.get(ROUNDED_STREAM)
+        if h is None:
+            if ctx.dtype == torch.float32:
+                return x
+            h = ops.round_rows(x, ctx.scratch("stream.rounded", (ctx.n_tokens, self.hidden)))
+        return h
+
+    def _sublayer(self, ctx, x, norm, result, pending):
+        rounded = ctx.scratch("stream.rounded", (ctx.n_tokens, self.hidden)) if ctx.dtype != torch.float32 else None
+        ops.add_normed(x, norm.weight, norm.eps, mult=self.mult, y=result if pending is None else None, add=pending,
+                       out=rounded)
+        ctx.shared[ROUNDED_STREAM] = rounded if rounded is not None else x
+
+    def forward(self, ctx, run, x, pending=None):
+        pending = fold_pending(x, pending)
+        result = ctx.scratch("sublayer.result", (ctx.n_tokens, self.hidden), torch.float32)
+        left = self.mixer.forward(ctx, run, self._rounded(ctx, x), result, accumulate=False)
+        self._sublayer(ctx, x, self.mixer_norm, result, left)
+        if self.ffn is not None:
+            left = self.ffn.forward(ctx, self._rounded(ctx, x), result, accumulate=False)
+            self._sublayer(ctx, x, self.ffn_norm, result, left)
+        return None
+
+
 class DepthMixedBlock(Block):
     """Pre-norm block whose sublayers read their normed input through a short causal convolution, with an
     optional per-layer token input, and whose output is a learned mix of every layer's result so far:

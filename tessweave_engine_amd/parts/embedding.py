@@ -114,8 +114,10 @@ class HashedPairEmbedding(TokenEmbedding):
 
 
 class OutputHead(Part):
-    def __init__(self, name, vocab, hidden, tied_to=None, suffix=".weight", scale=1.0):
-        """scale: a factor on the logits, applied to the float32 product."""
+    def __init__(self, name, vocab, hidden, tied_to=None, suffix=".weight", scale=1.0, softcap=None):
+        """scale: a factor on the logits, applied to the float32 product; softcap: the logits then pass
+        softcap * tanh(logit / softcap)."""
+        self.softcap = float(softcap) if softcap else 0.0
         self.name, self.vocab, self.hidden = name, int(vocab), int(hidden)
         self.suffix = suffix
         self.tied_to = tied_to
@@ -149,4 +151,6 @@ class OutputHead(Part):
         ops.linear(h, self.matrix(), logits)
         if self.scale != 1.0:
             ops.scale_values(logits, self.scale)
+        if self.softcap:
+            ops.softcap_values(logits, self.softcap)
         return logits

@@ -99,11 +99,16 @@ class GatedFeedForward(FeedForward):
         return None
 
 
-class ReluSquaredFeedForward(FeedForward):
-    """x += down( relu(up(h))^2 ): no gate, no biases. names = (up, down), the checkpoint prefixes of the two matrices."""
+class PlainFeedForward(FeedForward):
+    """x += down( act(up(h)) ): no gate, no biases; act "relu_squared" (max(z, 0)^2) or "gelu" (the exact one, z Phi(z)).
+    names = (up, down), the checkpoint prefixes of the two matrices. defer=False: the down projection always finishes
+    its sums itself (for a part that adds more to the same result)."""
 
-    def __init__(self, names, hidden, intermediate, suffix=".weight"):
+    def __init__(self, names, hidden, intermediate, suffix=".weight", activation="relu_squared", defer=True):
         up, down = names
+        if activation not in ops.LINEAR_ACTIVATIONS:
+            raise ValueError("a plain feed-forward computes relu_squared or gelu")
+        self.activation, self.defer = activation, bool(defer)
         self.hidden, self.intermediate = int(hidden), int(intermediate)
         self.up = Linear([up], hidden, [intermediate], suffixes=(suffix, ".bias"))
         self.down = Linear([down], intermediate, [hidden], suffixes=(suffix, ".bias"))
@@ -123,11 +128,18 @@ class ReluSquaredFeedForward(FeedForward):
         act = ctx.scratch("ffn.act", (n, self.intermediate))
         if n <= 64 and self.up.deferrable(n):
             # few rows: the product leaves its split-K sums, and the activation's kernel adds them up
-            ops.relu_squared(act, partial=self.up.forward_partials(ctx, h, "up"))
-        elif not self.up.forward_act(ctx, h, act, "relu_squared"):       # many rows: in the product's epilogue
+            ops.activation(act, self.activation, partial=self.up.forward_partials(ctx, h, "up"))
+        elif not self.up.forward_act(ctx, h, act, self.activation):       # many rows: in the product's epilogue
             self.up.forward(ctx, h, act)
-            ops.relu_squared(act)
-        if ctx.defer_sums and self.down.deferrable(n):
+            ops.activation(act, self.activation)
+        if self.defer and ctx.defer_sums and self.down.deferrable(n):
             return self.down.forward_partials(ctx, act, "down")          # whoever norms next adds them up
         self.down.forward(ctx, act, x, residual=x if accumulate else None)
         return None
+
+
+class ReluSquaredFeedForward(PlainFeedForward):
+    """x += down( relu(up(h))^2 )."""
+
+    def __init__(self, names, hidden, intermediate, suffix=".weight"):
+        super().__init__(names, hidden, intermediate, suffix=suffix, activation="relu_squared")

@@ -14,6 +14,12 @@ once a step (one product with [W_uk; W_uv] over the gathered key rows) into keys
 of their own, and the engine's ordinary prompt attention runs on those. A layer may read the cache slot of another
 layer (`LayerRun(writes_cache=False)`): it then has no down-projection of its own (`own_latent=False`) and uses that
 layer's c and kr with its own queries and its own W_uk, W_uv.
+
+Options: a learned sink per head (`sink_name`: exp(sink_a) more in head a's denominator, with no key and no value, not
+scaled; prompt portions then run the attention kernel that takes sinks), an output gate (`gate_name`: the heads'
+results times sigmoid(W_g h) before the output product), and a rotary encoding that pairs neighbouring elements: the
+rotated rows of W_q and of the down-projection are then reordered once, when the weights are bound, into the order
+that pairs element j with j + rot/2 (both sides of every score alike, so no score changes).
 """
 from __future__ import annotations
 
@@ -32,7 +38,7 @@ def _round_up(v, m):
 
 class LatentAttention(Mixer):
     def __init__(self, prefix, hidden, heads, dim, rot_dim, value_dim, latent, scale, position, eps, own_latent=True,
-                 names=("q", "dkv", "dkv.norm", "uk", "uv", "o")):
+                 names=("q", "dkv", "dkv.norm", "uk", "uv", "o"), sink_name=None, gate_name=None):
         """position: a rotary encoding over `rot_dim` elements (its `rotary_dim` may be smaller: the rest of the
         rotated part passes unchanged). scale multiplies the scores as given."""
         self.prefix, self.names = prefix, tuple(names)
@@ -40,8 +46,13 @@ class LatentAttention(Mixer):
         self.dim, self.rot_dim, self.value_dim, self.latent = int(dim), int(rot_dim), int(value_dim), int(latent)
         if min(self.heads, self.dim, self.rot_dim, self.value_dim, self.latent) <= 0:
             raise ValueError("heads and sizes must be positive")
-        if position.rotary_dim <= 0 or position.rotary_dim > self.rot_dim or position.pairing != "half":
-            raise ValueError("the rotated part needs a rotary encoding of at most rot_dim elements with the 'half' pairing")
+        if position.rotary_dim <= 0 or position.rotary_dim > self.rot_dim:
+            raise ValueError("the rotated part needs a rotary encoding of at most rot_dim elements")
+        self.sink_name = prefix + sink_name if sink_name else None
+        self.gate_name = prefix + gate_name if gate_name else None
+        if self.sink_name and self.heads > 32:
+            raise ValueError("the attention kernel that takes sinks holds up to 32 heads")
+        self.sink = None
         # sizes on the device: tails of zeros, which add nothing to a product
         self.dim_dev = _round_up(dim, 8)
         self.latent_dev, self.rot_dev = _round_up(latent, 16), _round_up(rot_dim, 16)
@@ -76,20 +87,36 @@ class LatentAttention(Mixer):
             specs += [TensorSpec(self._name(1), (L + R, C), MATRIX, NORMAL),
                       TensorSpec(self._name(2), (L,), VECTOR, ONE_PLUS_NORMAL)]
         specs += [TensorSpec(self._name(3), (H * D, L), MATRIX, NORMAL), TensorSpec(self._name(4), (H * E, L), MATRIX, NORMAL)]
+        if self.sink_name:
+            specs.append(TensorSpec(self.sink_name, (H,), VECTOR, NORMAL))
+        if self.gate_name:
+            specs.append(TensorSpec(self.gate_name, (H * E, C), MATRIX, NORMAL))
         return specs + self.o.tensor_specs()
 
     def bind(self, tensors, dtype, device):
         H, D, R, E, L = self.heads, self.dim, self.rot_dim, self.value_dim, self.latent
         Dp, Rp, Ep, Lp = self.dim_dev, self.rot_dev, self.value_dev, self.latent_dev
         q = tensors.pop(self._name(0)).view(H, D + R, self.hidden)
-        # one packed product: [all heads' unrotated query parts | all heads' rotated parts | latent | shared key part]
-        rows = [pad_groups(q[:, :D].reshape(H * D, -1), 0, D, Dp), pad_groups(q[:, D:].reshape(H * R, -1), 0, R, Rp)]
+        # An encoding that pairs neighbours (2j with 2j + 1): the rotated rows are put into the order that pairs j with
+        # j + rot/2, on the query side and the key side alike.
+        order = list(range(R))
+        if self.position.pairing == "adjacent":
+            rot = self.position.rotary_dim
+            order = list(range(0, rot, 2)) + list(range(1, rot, 2)) + list(range(rot, R))
+        turned = q[:, D:][:, order]
+        # one packed product: [all heads' unrotated query parts | all heads' rotated parts | latent | shared key part | gate]
+        rows = [pad_groups(q[:, :D].reshape(H * D, -1), 0, D, Dp), pad_groups(turned.reshape(H * R, -1), 0, R, Rp)]
         if self.own_latent:
             down = tensors.pop(self._name(1))
-            rows += [pad_groups(down[:L], 0, L, Lp), pad_groups(down[L:], 0, R, Rp)]
+            rows += [pad_groups(down[:L], 0, L, Lp), pad_groups(down[L:][order], 0, R, Rp)]
             self.latent_norm = tensors.pop(self._name(2)).contiguous()
-        packed = torch.cat(rows, 0).contiguous()
         self.q_col, self.c_col, self.kr_col = H * Dp, H * (Dp + Rp), H * (Dp + Rp) + Lp
+        self.g_col = sum(r.shape[0] for r in rows)
+        if self.gate_name:           # laid out like the heads' results
+            rows.append(pad_groups(tensors.pop(self.gate_name), 0, E, Ep))
+        if self.sink_name:
+            self.sink = tensors.pop(self.sink_name).contiguous()
+        packed = torch.cat(rows, 0).contiguous()
         self.proj_width = packed.shape[0]
         name = self.prefix + "packed"
         self.proj = Linear([name], self.hidden, [self.proj_width])
@@ -114,7 +141,7 @@ class LatentAttention(Mixer):
         self.position.bind(tensors, dtype, device)
 
     def weight_tensors(self):
-        return [t for t in (self.absorb, self.expand, self.latent_norm) if t is not None]
+        return [t for t in (self.absorb, self.expand, self.latent_norm, self.sink) if t is not None]
 
     def cache_need(self):
         return CacheNeed(paged=PagedKV(1, self.key_dev, None, self.latent_dev))
@@ -152,7 +179,7 @@ class LatentAttention(Mixer):
                 floats = ops.latent_decode_workspace_floats(nd, H, Lp, max(splits, ops.latent_decode_splits(nd, H, ctx.kv_capacity)))
                 ws = ctx.workspace.get("latent.split", (floats,), torch.float32)
             ops.latent_decode(q[:nd], keys, values, group.block_table, ctx.q_start, ctx.kv_len, nd, mixed, H, self.scale,
-                              splits=splits, workspace=ws)
+                              splits=splits, workspace=ws, sink=self.sink)
             ops.head_linear(mixed, Lp, self.expand, out[:nd], hd)
         if portions:
             # prompt portions: their sequences' cached latents expanded per head into pages of this step's own
@@ -165,12 +192,23 @@ class LatentAttention(Mixer):
             own_keys = ctx.workspace.get("latent.keys", (own_pages, H, page, hd), ctx.dtype)
             own_values = ctx.workspace.get("latent.values", (own_pages, H, hd, page), ctx.dtype)
             ops.latent_expand_store(up, rows, Lp, own_keys, own_values, H, self.dim, self.rot_dim, self.value_dim)
-            split = ops.attn_prefill_split(portions, H, H, longest_portion, ctx.max_kv_len)
-            ws = None
-            if split[0] > 1:
-                ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, hd, split[0]),), torch.float32)
-            ops.attn_prefill(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd,
-                             portions, longest_portion, out, H, H, hd, self.scale, split=split, workspace=ws)
+            if self.sink is not None:
+                splits = ops.attn_mixed_prefill_splits(n - nd, portions, ctx.max_kv_len)
+                ws = None
+                if splits > 1:
+                    floats = ops.attn_mixed_workspace_floats(portions, longest_portion, H, hd, splits)
+                    ws = ctx.workspace.get("latent.sink.split", (floats,), torch.float32)
+                ops.attn_mixed(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd, portions, longest_portion,
+                               out, H, H, self.scale, sink=self.sink, splits=splits, workspace=ws)
+            else:
+                split = ops.attn_prefill_split(portions, H, H, longest_portion, ctx.max_kv_len)
+                ws = None
+                if split[0] > 1:
+                    ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, hd, split[0]),), torch.float32)
+                ops.attn_prefill(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd,
+                                 portions, longest_portion, out, H, H, hd, self.scale, split=split, workspace=ws)
+        if self.gate_name:
+            ops.sigmoid_gate(out, proj[:, self.g_col:self.g_col + H * hd])
         if ctx.defer_sums and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # whoever norms next adds them up
         self.o.forward(ctx, out, x, residual=x if accumulate else None)
