@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(LatentFinishArgs a) 
       const int head = i / a.hd, d = i % a.hd;
       T v = tw_from_float<T>(0.f);
       if (d < a.D) v = row[head * a.Dp + d];                                   // (the unrotated parts lie first in the row)
-      else if (d < a.D + a.rot) v = q[(size_t)head * K + a.Lp + d - a.D];
+      else if (d < a.D + a.Rp) v = q[(size_t)head * K + a.Lp + d - a.D];     // (turned or not; zeros behind the part's own size)
       qf[i] = v;
     }
   }
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(LatentFinishArgs a) 
       float other;
       lt_rotate_pair(tw_to_float(src[d - half]), tw_to_float(src[d]), cs[d - half], sn[d - half], other, v);
     } else {
-      v = 0.f;
+      v = tw_to_float(src[d]);                   // what the encoding does not turn passes (the padding behind it is zeros)
     }
     key[a.Lp + d] = tw_from_float<T>(v);
   }
@@ -111,7 +111,7 @@ extern "C" int tw_latent_finish(int dtype, const void* proj, long ld, int q_col,
   TW_REQUIRE(q_col >= 0 && ld >= q_col + (long)H * Rp && ld_q >= (long)H * (Lp + Rp) && Lp >= 0);
   if (keys) {
     TW_REQUIRE(values && slots && norm_w && L > 0 && Lp >= L && page_size > 0 && eps > 0.f);
-    TW_REQUIRE(c_col >= 0 && kr_col >= 0 && ld >= c_col + (long)L && ld >= kr_col + (long)rot);
+    TW_REQUIRE(c_col >= 0 && kr_col >= 0 && ld >= c_col + (long)L && ld >= kr_col + (long)Rp);
   }
   if (n == 0) return 0;
   LatentFinishArgs a{proj, ld, q_col, c_col, kr_col, cos_t, sin_t, norm_w, q_out, ld_q, q_full, ld_full, D, Dp, hd, full_from,

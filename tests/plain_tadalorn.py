@@ -33,11 +33,12 @@ def silu(z):
 
 def rotate_pairs(x, positions, dims, base):
     """x [T, heads, >= dims]: of the first `dims` elements of a head, element 2i turns with element 2i + 1 by the
-    angle position * base^(-2i / dims); the rest pass."""
+    angle position * base^(-2i / dims); the rest pass. (A float32 run rounds the frequencies and the angles to
+    float32: a thousand tokens in, an angle of hundreds of radians is then off by some 1e-5.)"""
     half = dims // 2
-    f = float(base) ** (-2.0 * torch.arange(half, dtype=torch.float64) / dims)
-    angle = positions.to(torch.float64).view(-1, 1, 1) * f.view(1, 1, -1)
-    cos, sin = torch.cos(angle).to(x.dtype), torch.sin(angle).to(x.dtype)
+    f = (float(base) ** (-2.0 * torch.arange(half, dtype=torch.float64) / dims)).to(x.dtype)
+    angle = positions.to(x.dtype).view(-1, 1, 1) * f.view(1, 1, -1)          # in the working precision, as everything
+    cos, sin = torch.cos(angle), torch.sin(angle)
     u, v = x[..., 0:dims:2], x[..., 1:dims:2]
     turned = torch.stack([u * cos - v * sin, v * cos + u * sin], -1).flatten(-2)
     return torch.cat([turned, x[..., dims:]], -1)
@@ -150,19 +151,30 @@ def plain_expert(h, up, down):
     return gelu_erf(h @ up.T) @ down.T
 
 
-def routed_ff(h, w, mlp):
+def router_margin(z, top):
+    """Per token, how far the last chosen logit lies above the best one left out (infinite if all are chosen)."""
+    if top >= z.shape[-1]:
+        return torch.full(z.shape[:-1], math.inf, dtype=z.dtype)
+    best = torch.topk(z, top + 1, dim=-1).values
+    return best[..., top - 1] - best[..., top]
+
+
+def routed_ff(h, w, mlp, margins=None):
     """Every token runs the `top` experts with the largest router logits, weighted by the softmax over those logits
     alone, and the shared expert if there is one."""
     T = h.shape[0]
     top = mlp["router"]["top"]
     z = h @ w["router"].T + w["router.b"]
+    if margins is not None:
+        margins.append(router_margin(z, top))
     best, ids = torch.topk(z, top, dim=-1)
     p = torch.softmax(best, -1)
     out = torch.zeros_like(h)
-    for t in range(T):
-        for r in range(top):
-            e = int(ids[t, r])
-            out[t] = out[t] + p[t, r] * plain_expert(h[t:t + 1], w[f"e{e}.up"], w[f"e{e}.down"])[0]
+    for e in range(z.shape[-1]):
+        share = (p * (ids == e)).sum(-1)                  # a token's weight for expert e, zero if it did not choose it
+        rows = torch.nonzero((ids == e).any(-1)).flatten()
+        if len(rows):
+            out[rows] = out[rows] + share[rows, None] * plain_expert(h[rows], w[f"e{e}.up"], w[f"e{e}.down"])
     if mlp.get("shared") is not None:
         out = out + plain_expert(h, w["shared.up"], w["shared.down"])
     return out
@@ -176,9 +188,9 @@ def sub(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(config, weights, tokens, dtype=torch.float64, layers_out=None):
+def forward(config, weights, tokens, dtype=torch.float64, layers_out=None, margins=None):
     """Logits [T, V] of a whole sequence. weights: name -> tensor (any float type). layers_out: a list that gets the
-    stream after every layer."""
+    stream after every layer; margins: a list that gets every routed layer's `router_margin` per token."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps, mult = config["norm"]["eps"], config["residual_mult"]
     x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
@@ -189,7 +201,7 @@ def forward(config, weights, tokens, dtype=torch.float64, layers_out=None):
         x = x + mult * rms_norm(y, w[p + "norm1"], eps)
         mlp = layer.get("mlp")
         if mlp is not None:
-            y = dense_ff(x, sub(w, p + "mlp.")) if mlp["kind"] == "dense" else routed_ff(x, sub(w, p + "mlp."), mlp)
+            y = dense_ff(x, sub(w, p + "mlp.")) if mlp["kind"] == "dense" else routed_ff(x, sub(w, p + "mlp."), mlp, margins)
             x = x + mult * rms_norm(y, w[p + "norm2"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())

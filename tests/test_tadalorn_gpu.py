@@ -1,0 +1,675 @@
+"""The Tadalorn design on the GPU against the plain implementation (`plain_tadalorn.py`).
+
+Mechanisms alone (each kernel against the plain function of the same mechanism: the norm on a sublayer's result, the
+soft cap, the exact gelu, the output gate, whole-row norms with the rotation of pairs, the window with kept first keys
+and a sink, made sharp so that one key just inside or just outside an edge carries the row, the router with a bias and
+the softmax over the chosen, the grouped experts without a gate, the mLSTM walked and in chunks over cut sequences in
+reused slots), then each mixer alone in a model of one layer, then whole models through the package's loader, cache
+manager and step function: prefill against token-by-token decoding, portions down to two tokens, unequal batches
+against each request alone, few pages and slots that are freed and used again, attention made sharp over a long
+prompt, a state that must survive hundreds of tokens, long decoding from HIP graphs, sizes drawn at random, and greedy
+generation through the scheduler.
+
+Bars: float32 rows must agree with the float64 plain implementation to 2e-5 of the logits' spread (the kernels sum
+in other orders) plus three times what the PLAIN implementation run in float32 is off by in that row. The mLSTM divides
+by max(|n . q|, exp(-m)), and where the sum n . q nearly cancels, float32 arithmetic itself, in any order of
+operations, moves the row: one row in fifty may therefore lie beyond that, none beyond 1e-3 (a lost key, state or
+window edge moves a row by 1e-2 and more). bfloat16 rows must agree to 3 % of the spread, one in five up to three times
+as far (the narrow models here round coarsely). A token whose router logits nearly tie between the last expert chosen
+and the next (`plain.router_margin` under CLOSE) may go the other way in bfloat16, and what it leaves in the recurrent
+states and the caches reaches every later row of its sequence: rows behind a sequence's first such token are only held
+to a typical error within five times the bar. Every kernel that runs in bfloat16 is the same template as in float32.
+"""
+import math
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import plain_tadalorn as plain
+from tadalorn_util import (CONFIGS, Driver, attention, config, dense, latent, make_weights, mlstm, moe, row_error, same_as,
+                           write_folder)
+
+pytestmark = pytest.mark.gpu
+
+BAR = {"float32": 2e-5, "bfloat16": 3e-2}
+CLOSE = 0.1
+LENGTHS = {"odd": (61, 23, 9, 150, 1), "wide": (70, 12, 33, 101, 2), "one": (40, 7, 90)}
+
+
+def double(weights):
+    return {k: v.double() for k, v in weights.items()}
+
+
+class Slack(np.ndarray):
+    """Router margins per row that also carry, as `.float32`, what the plain implementation in float32 is off by."""
+
+
+def reference(c, weights, toks):
+    """(logits [T, V] in float64, per token the smallest router margin with the float32 slack per row on it)."""
+    margins = []
+    logits = plain.forward(c, double(weights), toks, margins=margins).numpy()
+    least = torch.stack(margins).min(0).values.numpy() if margins else np.full(len(toks), np.inf)
+    least = np.asarray(least, dtype=np.float64).view(Slack)
+    single = plain.forward(c, {k: v.float() for k, v in weights.items()}, toks, dtype=torch.float32).numpy()
+    least.float32 = row_error(single, logits)
+    return logits, least
+
+
+def tdtype(name):
+    return getattr(torch, name)
+
+
+def ints(values, device):
+    return torch.tensor(values, dtype=torch.int32, device=device)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# mechanisms alone
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,C,splits", [(5, 88, 0), (70, 1000, 3), (3, 4097, 0), (2, 20000, 2), (4, 4096, 0)])
+def test_norm_on_a_result_added_into_the_stream(device, dtype, n, C, splits):
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(n + C)
+    x = torch.randn(n, C, generator=g).to(device)
+    w = (1.0 + 0.3 * torch.randn(C, generator=g)).to(device)
+    parts = torch.randn(max(splits, 1), n, C, generator=g).to(device) * 3.0
+    y = parts.sum(0)
+    want = x.double() + 0.6 * plain.rms_norm(y.double(), w.double(), 1e-5)
+    out = torch.empty(n, C, dtype=tdtype(dtype), device=device)
+    got = x.clone()
+    if splits:
+        ops.add_normed(got, w, 1e-5, mult=0.6, add=parts.contiguous(), out=out)
+    else:
+        ops.add_normed(got, w, 1e-5, mult=0.6, y=y, out=out)
+    assert torch.allclose(got.double(), want, atol=2e-5, rtol=1e-5)
+    assert torch.equal(out, got.to(tdtype(dtype)))
+
+
+def test_soft_cap_gelu_and_output_gate(device):
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(7, 333, generator=g) * 20).to(device)
+    got = ops.softcap_values(x.clone(), 15.0)
+    assert torch.allclose(got.double(), 15.0 * torch.tanh(x.double() / 15.0), atol=1e-5)
+    z = (torch.randn(9, 70, generator=g) * 3).to(device)
+    assert torch.allclose(ops.activation(z.clone(), "gelu").double(), plain.gelu_erf(z.double()), atol=1e-6)
+    parts = torch.randn(3, 9, 70, generator=g).to(device)
+    got = ops.activation(torch.empty(9, 70, device=device), "gelu", partial=parts)
+    assert torch.allclose(got.double(), plain.gelu_erf(parts.sum(0).double()), atol=1e-6)
+    for dtype in (torch.float32, torch.bfloat16):
+        o = torch.randn(9, 80, generator=g).to(device).to(dtype)
+        wide = torch.randn(9, 200, generator=g).to(device)                  # the gate: columns 40 .. 120 of wider rows
+        got = ops.sigmoid_gate(o.clone(), wide[:, 40:120])
+        want = o.double() * torch.sigmoid(wide[:, 40:120].double())
+        assert torch.allclose(got.double(), want, atol=1e-6 if dtype == torch.float32 else 2e-2)
+
+
+def paged(k, v, page, order_seed, device, dtype, dim_dev):
+    """Dense k, v [T, G, D] into pages handed out in an order of their own: (keys [pages, G, page, dim_dev], values
+    [pages, G, dim_dev, page], block table row, slots per token)."""
+    T, G, D = k.shape
+    blocks = (T + page - 1) // page
+    order = list(range(blocks + 3))
+    random.Random(order_seed).shuffle(order)
+    table = order[:blocks]
+    keys = torch.full((blocks + 3, G, page, dim_dev), float("nan"), dtype=dtype, device=device)
+    values = torch.full((blocks + 3, G, dim_dev, page), float("nan"), dtype=dtype, device=device)
+    slots = [table[t // page] * page + t % page for t in range(T)]
+    return keys, values, table, slots
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,D,rot,window,keep,page", [(4, 2, 24, 16, 9, 3, 4), (8, 8, 32, 32, 64, 0, 16), (4, 1, 64, 32, 5, 20, 8),
+                                                        (2, 2, 16, 0, 33, 1, 16), (6, 3, 40, 8, 16, 16, 4), (3, 3, 128, 128, 40, 4, 16)])
+def test_window_with_kept_first_keys_and_a_sink_made_sharp(device, dtype, H, G, D, rot, window, keep, page):
+    """Whole-row norms, rotation of pairs, cache write and the attention kernel, against the plain softmax over the
+    plain mask. Every query row is made to point at ONE key with a large score: the key just inside its window, the one
+    just outside, the last kept key, the first one not kept, the first token, itself. A key seen wrongly or lost moves
+    its row by the size of a value. A prompt portion behind a cached history, then single tokens."""
+    from tessweave_engine_amd.kernels import ops
+    T, eps, scale = 150, 1e-5, 0.5
+    g = torch.Generator().manual_seed(H * D + window)
+    Dp = (D + 15) // 16 * 16
+    targets = []
+    for i in range(T):
+        choice = [i - window + 1, i - window, keep - 1, keep, 0, i][i % 6]
+        targets.append(min(max(choice, 0), i))
+    # rows before the norms: k random; q of position i a multiple of what makes its rotated self meet key targets[i]
+    k_raw = torch.randn(T, G * D, generator=g).double()
+    wq, wk = (1.0 + 0.2 * torch.randn(H * D, generator=g)).double(), (1.0 + 0.2 * torch.randn(G * D, generator=g)).double()
+    pos = torch.arange(T)
+    k_fin = plain.rms_norm(k_raw, wk, eps).view(T, G, D)
+    k_rot = plain.rotate_pairs(k_fin, pos, rot, 100.0) if rot else k_fin
+    q_want = torch.stack([k_rot[targets[i]].repeat_interleave(H // G, 0) for i in range(T)]) * 3.0        # [T, H, D], rotated
+    q_fin = plain.rotate_pairs(q_want, -pos, rot, 100.0) if rot else q_want                                 # turned back
+    q_raw = (q_fin.reshape(T, H * D) / wq) + 0.05 * torch.randn(T, H * D, generator=g).double()
+    src = torch.cat([q_raw, k_raw], 1).float().to(device)
+    # the plain result from the same float32 rows
+    s64 = src.double().cpu()
+    qn = plain.rms_norm(s64[:, :H * D], wq, eps).view(T, H, D)
+    kn = plain.rms_norm(s64[:, H * D:], wk, eps).view(T, G, D)
+    if rot:
+        qn, kn = plain.rotate_pairs(qn, pos, rot, 100.0), plain.rotate_pairs(kn, pos, rot, 100.0)
+    vn = s64[:, H * D:].view(T, G, D)
+    visible = plain.window_mask(T, window, keep)
+    want = torch.zeros(T, H, D, dtype=torch.float64)
+    for a in range(H):
+        p = plain.softmax_with_sink(qn[:, a] @ kn[:, a // (H // G)].T * scale, visible, torch.zeros((), dtype=torch.float64))
+        want[:, a] = p @ vn[:, a // (H // G)]
+    # the kernels
+    dt = tdtype(dtype)
+    keys, values, table, slots = paged(kn, vn, page, 3, device, dt, Dp)
+    half = rot // 2
+    if rot:
+        f = 100.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / rot)
+        ang = pos.double().view(-1, 1) * f
+        cos, sin = torch.cos(ang).float().to(device).contiguous(), torch.sin(ang).float().to(device).contiguous()
+    else:
+        cos = sin = None
+    q = torch.empty(T, H * Dp, dtype=dt, device=device)
+    ops.qk_finish(src, 0, H * D, wq.float().to(device), wk.float().to(device), cos, sin, q, keys, values, ints(slots, device),
+                  H, G, D, rot, eps, adjacent=True)
+    sink = torch.zeros(H, device=device)
+    out = torch.full((T, H * Dp), float("nan"), dtype=dt, device=device)
+    width = len(table) + 2
+    bt = ints([table + [-1] * (width - len(table))], device)
+    first = 100                                              # a portion of 100 - 37 tokens behind 37 cached ones, then single tokens
+    for lo, hi in [(0, 37), (37, first)] + [(t, t + 1) for t in range(first, T)]:
+        ops.attn_mixed(q[lo:hi], keys, values, bt, ints([0, hi - lo], device), ints([hi], device), 0, 1, hi - lo, out[lo:hi], H, G,
+                       scale, window=window, keep_first=keep, sink=sink)
+    got = out.view(T, H, Dp)[:, :, :D].double().cpu()
+    assert torch.isfinite(out.view(T, H, Dp)[:, :, :D]).all()
+    tol = 1e-4 if dtype == "float32" else 6e-2
+    err = (got - want).abs().amax((1, 2))
+    assert err.max() < tol, (int(err.argmax()), targets[int(err.argmax())], float(err.max()))
+    # the test would see an edge that is off by one: the plain result for a window one longer differs
+    other = plain.window_mask(T, window + 1, keep)
+    moved = 0
+    for a in range(H):
+        p = plain.softmax_with_sink(qn[:, a] @ kn[:, a // (H // G)].T * scale, other, torch.zeros((), dtype=torch.float64))
+        moved = max(moved, float(((p @ vn[:, a // (H // G)]) - want[:, a]).abs().max()))
+    assert moved > 10 * tol
+
+
+@pytest.mark.parametrize("C,X,top", [(72, 70, 4), (90, 7, 3), (64, 1, 1), (2048, 16, 2), (88, 5, 5)])
+def test_router_with_bias_and_softmax_over_the_chosen(device, C, X, top):
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(C + X)
+    n = 37
+    h = torch.randn(n, C, generator=g).to(device)
+    router = (torch.randn(X, C, generator=g) / math.sqrt(C)).to(device)
+    bias = torch.randn(X, generator=g).to(device)
+    if X > 2:
+        router[2] = router[1]
+        bias[2] = bias[1]                                       # a tie: the lower index wins
+    ids = torch.empty(n, top, dtype=torch.int32, device=device)
+    weights = torch.empty(n, top, device=device)
+    ops.moe_route(h, router, top, ids, weights, bias=bias, weighting="softmax_chosen")
+    z = h.double() @ router.double().T + bias.double()
+    best, want_ids = torch.topk(z, top, dim=-1)
+    assert torch.allclose(weights.double(), torch.softmax(best, -1), atol=1e-5)
+    assert torch.allclose(torch.gather(z, 1, ids.long()), best, atol=1e-5)
+    if X > 2:
+        chosen = ids.long()
+        both = (chosen == 1).any(-1) ^ (chosen == 2).any(-1)
+        assert not (chosen[both] == 2).any()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,C,X,top,F", [(1, 88, 5, 2, 40), (9, 128, 16, 4, 64), (300, 96, 3, 3, 24), (130, 72, 64, 1, 100), (17, 64, 2, 1, 32)])
+def test_grouped_experts_without_a_gate(device, dtype, n, C, X, top, F):
+    from tessweave_engine_amd.kernels import ops
+    dt = tdtype(dtype)
+    g = torch.Generator().manual_seed(n + X)
+    h = torch.randn(n, C, generator=g).to(device).to(dt)
+    ups = (torch.randn(X, F, C, generator=g) / math.sqrt(C)).to(dt)
+    downs = (torch.randn(X, C, F, generator=g) / math.sqrt(F)).to(dt)
+    ids = torch.stack([torch.randperm(X, generator=g)[:top] for _ in range(n)]).to(torch.int32).to(device)
+    weights = torch.softmax(torch.randn(n, top, generator=g), -1).to(device)
+    Cd, Fd = ops.moe_pad(C), ops.moe_pad(F)
+    up = torch.zeros(X, Fd, Cd, dtype=dt, device=device)
+    down = torch.zeros(X, C, Fd, dtype=dt, device=device)
+    up[:, :F, :C] = ups.to(device)
+    down[:, :, :F] = downs.to(device)
+    store = {}
+
+    def scratch(tag, shape, dtype_):
+        store[tag] = torch.empty(shape, dtype=dtype_, device=device)
+        return store[tag]
+    want = torch.zeros(n, C, dtype=torch.float64)
+    for t in range(n):
+        for r in range(top):
+            e = int(ids[t, r])
+            want[t] += weights[t, r].double().cpu() * plain.plain_expert(h[t:t + 1].double().cpu(), ups[e].double(), downs[e].double())[0]
+    base = torch.randn(n, C, generator=g).to(device)
+    for accumulate in (True, False):
+        x = base.clone()
+        ops.moe_experts(h, ids, weights, None, ops.moe_blocked(up), ops.moe_blocked(down), 0.0, x, scratch, kind="gelu",
+                        accumulate=accumulate)
+        got = x.double().cpu() - (base.double().cpu() if accumulate else 0.0)
+        assert torch.allclose(got, want, atol=2e-5 if dtype == "float32" else 4e-2), accumulate
+
+
+def mlstm_plain_heads(proj, H, D, E, i_b, f_b, cap):
+    T = proj.shape[0]
+    p = proj.double().cpu()
+    q = p[:, :H * D].view(T, H, D) * D ** -0.5
+    k = p[:, H * D:2 * H * D].view(T, H, D)
+    v = p[:, 2 * H * D:2 * H * D + H * E].view(T, H, E)
+    i_log = cap * torch.tanh((p[:, -2 * H:-H] + i_b.double().cpu()) / cap)
+    f_log = torch.nn.functional.logsigmoid(cap * torch.tanh((p[:, -H:] + f_b.double().cpu()) / cap))
+    return torch.stack([plain.mlstm_steps(q[:, a], k[:, a], v[:, a], i_log[:, a], f_log[:, a]) for a in range(H)], 1).reshape(T, H * E)
+
+
+@pytest.mark.parametrize("walk", [True, False], ids=["walked", "chunks"])
+@pytest.mark.parametrize("H,D,E", [(3, 20, 24), (1, 13, 10), (2, 128, 64), (4, 32, 80), (2, 256, 16), (1, 64, 200)])
+def test_mlstm_over_cut_sequences_in_reused_slots(device, H, D, E, walk):
+    """Three sequences cut differently (one whole, one in portions of 1, 2, 5 and 33 tokens, one token by token), their
+    states in slots that other sequences used before; gates that meet their cap and forget gates near one."""
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(H * D + E)
+    cap = 6.0
+    lengths = [70, 59, 23]
+    width = 2 * H * D + H * E + 2 * H
+    Dp, Ep = (D + 15) // 16 * 16, (E + 15) // 16 * 16
+    i_b, f_b = torch.randn(H, generator=g).to(device), (3.0 + torch.randn(H, generator=g)).to(device)
+    S = torch.randn(4, H, Ep, Dp, generator=g).to(device)           # slots hold what others left: opened states are zeroed below
+    n_st = torch.randn(4, 2, H, Dp, generator=g).to(device)
+    m_st = torch.randn(4, 2, H, generator=g).to(device)
+    seqs = []
+    for s, T in enumerate(lengths):
+        proj = torch.randn(T, width, generator=g)
+        proj[:, -2 * H:] *= 4.0
+        seqs.append(proj.to(device))
+    wants = [mlstm_plain_heads(p, H, D, E, i_b, f_b, cap) for p in seqs]
+    cuts = [[70], [1, 2, 5, 33, 1, 2, 5, 10], [1] * 23]
+    slots = [2, 0, 3]
+    for s in slots:
+        S[s].zero_(); n_st[s].zero_(); m_st[s].zero_()
+    at, steps = [0, 0, 0], [0, 0, 0]
+    outs = [torch.zeros(T, H * E, device=device) for T in lengths]
+    while any(cuts):
+        rows, q_start, sl, ph, who = [], [0], [], [], []
+        for s in range(3):
+            if cuts[s]:
+                n = cuts[s].pop(0)
+                rows.append(seqs[s][at[s]:at[s] + n])
+                q_start.append(q_start[-1] + n)
+                sl.append(slots[s]); ph.append(steps[s] & 1); who.append((s, at[s], n))
+                at[s] += n; steps[s] += 1
+        proj = torch.cat(rows).contiguous()
+        out = torch.full((proj.shape[0], H * E), float("nan"), device=device)
+        ops.mlstm(proj, 0, H * D, 2 * H * D, width - 2 * H, width - H, i_b, f_b, S, n_st, m_st, ints(q_start, device), ints(sl, device),
+                  ints(ph, device), 0, len(sl), out, H, D, E, D ** -0.5, cap, walk)
+        for j, (s, lo, n) in enumerate(who):
+            outs[s][lo:lo + n] = out[q_start[j]:q_start[j + 1]]
+    for s in range(3):
+        want = wants[s]
+        err = (outs[s].double().cpu() - want).abs().max() / want.abs().max()
+        assert err < 5e-5, (s, float(err))          # (float32 sums in another order than the plain float64 walk)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# whole models
+
+@pytest.fixture(scope="module", params=list(CONFIGS))
+def model(request, tmp_path_factory, device):
+    name = request.param
+    c = CONFIGS[name]
+    weights = make_weights(c, seed=len(name))
+    folder = write_folder(tmp_path_factory.mktemp("tadalorn_" + name), c, weights)
+    g = torch.Generator().manual_seed(50 + len(name))
+    tokens = {f"r{i}": torch.randint(0, c["vocab"], (n,), generator=g).tolist() for i, n in enumerate(LENGTHS[name])}
+    both = {rid: reference(c, weights, toks) for rid, toks in tokens.items()}
+    return dict(name=name, config=c, weights=weights, folder=folder, tokens=tokens, want={k: v[0] for k, v in both.items()},
+                margin={k: v[1] for k, v in both.items()})
+
+
+def check_rows(err, dtype, what="", margin=None):
+    """ERR: one relative error per row of ONE sequence (or of several, without margins)."""
+    err = np.asarray(err)
+    assert np.isfinite(err).all(), what
+    if dtype == "bfloat16":
+        margin = np.full(len(err), np.inf) if margin is None else np.asarray(margin)
+        behind = np.cumsum(margin < CLOSE) > 0                     # rows that may have read what a close call left
+        sure, rest = err[~behind], err[behind]
+        if len(sure):
+            assert sure.max() < 3 * BAR[dtype], (what, int(sure.argmax()), float(sure.max()))
+            assert (sure > BAR[dtype]).sum() <= max(1, len(sure) // 5), (what, np.nonzero(sure > BAR[dtype])[0].tolist())
+            assert np.median(sure) < BAR[dtype], (what, float(np.median(sure)))
+        if len(rest):
+            assert np.median(rest) < 5 * BAR[dtype], (what, float(np.median(rest)))
+    else:
+        allowed = BAR[dtype] + 3.0 * getattr(margin, "float32", 0.0)
+        assert err.max() < 50 * BAR[dtype], (what, int(err.argmax()), float(err.max()))
+        assert (err >= allowed).sum() <= max(1, len(err) // 50), (what, np.nonzero(err >= allowed)[0].tolist())
+
+
+def check_all(model, got, dtype, only=None):
+    for rid, want in model["want"].items():
+        if only is not None and rid not in only:
+            continue
+        assert np.isfinite(got[rid]).all()
+        check_rows(row_error(got[rid], want), dtype, rid, model["margin"][rid])
+
+
+ONE_LAYER = {
+    "attention": attention(4, 2, 24, 16, 0.3, 3, 11, 2, base=100.0),
+    "attention_no_keep_one_tap": attention(2, 2, 16, 16, 0.25, 1, 7, 0),
+    "latent": latent(3, 24, 8, 40, 48, 0.2, base=500.0),
+    "latent_large": latent(2, 40, 24, 96, 250, 0.1),             # a latent too large for the one-head kernel
+    "mlstm": mlstm(3, 20, 24, 8.0),
+    "dense": dict(mlstm(1, 16, 16, 4.0), mlp=dense(72)),
+    "experts": dict(mlstm(1, 16, 16, 4.0), mlp=moe(7, 3, 40, shared=24)),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", list(ONE_LAYER))
+def test_each_mechanism_alone_in_a_model_of_one_layer(device, tmp_path, kind, dtype):
+    """One layer, whole and then cut (portions, single tokens, beside another request), pages of four tokens."""
+    c = config([ONE_LAYER[kind]], width=72, vocab=120, mult=0.8, softcap=12.0)
+    weights = make_weights(c, seed=3)
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(1)
+    tokens = {"a": torch.randint(0, 120, (75,), generator=g).tolist(), "b": torch.randint(0, 120, (19,), generator=g).tolist()}
+    want = {k: reference(c, weights, v) for k, v in tokens.items()}
+    d = Driver(folder, dtype, pages=60, page_size=4, max_requests=2)
+    whole = d.run([[("a", 75), ("b", 19)]], tokens)
+    cut = d.run([[("a", 33)], [("a", 2), ("b", 5)], [("a", 17), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 13 + [[("a", 10)]], tokens)
+    for got in (whole, cut):
+        for k in tokens:
+            check_rows(row_error(got[k], want[k][0]), dtype, (kind, k), want[k][1])
+    d.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_prompts(model, dtype):
+    d = Driver(model["folder"], dtype, pages=40, page_size=8)
+    got = d.run([[(rid, len(toks))] for rid, toks in model["tokens"].items()], model["tokens"])
+    check_all(model, got, dtype)
+    d.close()
+
+
+def test_stream_after_every_layer(model):
+    """float32: the residual stream after each layer (one that runs with another's weights included) against the plain one's."""
+    from tessweave_engine_amd.engine.step import StepEntry
+    rid = "r0"
+    toks = model["tokens"][rid]
+    want = []
+    plain.forward(model["config"], double(model["weights"]), toks, layers_out=want)
+    d = Driver(model["folder"], "float32", pages=24, page_size=8, graphs=False)
+    seq = d.cache.open(rid)
+    ctx, ordered, _ = d.stepper.prepare([StepEntry(seq, list(toks), [len(toks) - 1])])
+    seen = []
+    ctx.segment_end = lambda i: seen.append(ctx.scratch("residual", (ctx.n_tokens, model["config"]["width"]), torch.float32).clone())
+    with torch.cuda.stream(d.stepper.stream):
+        d.stepper.upload(ctx)
+        d.model.forward(ctx)
+    d.stepper.synchronize()
+    d.stepper.finish(ordered)
+    assert len(seen) == len(want)
+    for i, (got, ref) in enumerate(zip(seen, want)):
+        assert torch.allclose(got.cpu().double(), ref, atol=2e-5 * max(1.0, ref.abs().max().item())), i
+    d.close()
+
+
+@pytest.mark.parametrize("dtype,graphs", [("float32", True), ("float32", False), ("bfloat16", True)])
+def test_token_by_token(model, dtype, graphs):
+    """Every token decoded alone from the first on (the first tokens of a sequence included)."""
+    rid = "r0"
+    d = Driver(model["folder"], dtype, pages=24, page_size=4, graphs=graphs)
+    got = d.run([[(rid, 1)] for _ in model["tokens"][rid]], model["tokens"])
+    check_all(model, got, dtype, only=[rid])
+    if graphs:
+        assert d.model.graph_safe_model and d.stepper.graph_replays > 0
+    d.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("sizes", [[2], [3, 1, 2], [16, 5, 2, 2, 9], [7, 8, 1], [17, 32]])
+def test_portions(model, dtype, sizes):
+    rid = max(model["tokens"], key=lambda r: len(model["tokens"][r]))
+    total, schedule, i = len(model["tokens"][rid]), [], 0
+    while total:
+        n = min(sizes[i % len(sizes)], total)
+        schedule.append([(rid, n)])
+        total -= n
+        i += 1
+    d = Driver(model["folder"], dtype, pages=50, page_size=4)
+    got = d.run(schedule, model["tokens"])
+    check_all(model, got, dtype, only=[rid])
+    d.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [0, 1])
+def test_unequal_batches_few_pages_two_slots(model, dtype, seed):
+    """Portions of some requests beside single tokens of others; at most two requests live, so that every state slot
+    is used again (mLSTM states, convolution inputs), and a page pool that only just holds them."""
+    rng = random.Random(seed)
+    tokens = model["tokens"]
+    pending, live, schedule = list(tokens), {}, []
+    while pending or live:
+        while pending and len(live) < 2:
+            rid = pending.pop(0)
+            live[rid] = dict(left=len(tokens[rid]), prompt=rng.randrange(1, len(tokens[rid]) + 1))
+        parts = []
+        for rid, r in list(live.items()):
+            if len(live) > 1 and rng.random() < 0.25:
+                continue
+            n = min(r["left"], rng.choice([2, 3, 5, 11, 16]) if r["prompt"] > 0 else 1)
+            r["prompt"] -= n
+            r["left"] -= n
+            parts.append((rid, n))
+            if r["left"] == 0:
+                del live[rid]
+        if parts:
+            schedule.append(parts)
+    page = 8
+    longest = sorted(len(t) for t in tokens.values())[-2:]
+    pages = sum((n + page - 1) // page for n in longest)
+    d = Driver(model["folder"], dtype, pages=pages, page_size=page, max_requests=2)
+    got = d.run(schedule, tokens)
+    check_all(model, got, dtype)
+    d.close()
+
+
+def test_ways_of_cutting_agree(model):
+    """float32: whole, token by token and in portions beside another request differ by rounding only."""
+    tokens = model["tokens"]
+    rid, other = "r0", "r2"
+    runs = []
+    for schedule in ([[(rid, len(tokens[rid]))]],
+                     [[(rid, 1)] for _ in tokens[rid]],
+                     [[(other, 1), (rid, 5)]] + [[(rid, 2), (other, 1)] for _ in range(500)]):
+        d = Driver(model["folder"], "float32", pages=50, page_size=4)
+        fixed, used = [], {}
+        for parts in schedule:
+            parts = [(r, min(n, len(tokens[r]) - used.get(r, 0))) for r, n in parts]
+            parts = [(r, n) for r, n in parts if n > 0]
+            for r, n in parts:
+                used[r] = used.get(r, 0) + n
+            if parts:
+                fixed.append(parts)
+        runs.append(d.run(fixed, tokens)[rid])
+        d.close()
+    for other_run in runs[1:]:
+        check_rows(row_error(other_run, runs[0]), "float32", "cuts", model["margin"][rid])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["odd", "wide"])
+def test_sharp_attention_over_a_long_prompt(device, tmp_path, dtype, name):
+    """Scores eight times as large: every softmax sits on one or two keys, wherever they lie among hundreds (far back,
+    at a page's edge, a kept first token, the window's last). 600 tokens: 330 in one step, then portions of 64, 15, 2
+    and single tokens, on pages of four tokens handed out in an order of their own. float32 rows must agree to 1e-3,
+    where a key that is lost or seen wrongly moves a row by a tenth and more; in bfloat16 the typical row must stay
+    within the bar."""
+    c = CONFIGS[name]
+    weights = make_weights(c, seed=13, sharp=8.0 if dtype == "float32" else 2.0)
+    folder = write_folder(tmp_path, c, weights)
+    toks = torch.randint(0, c["vocab"], (600,), generator=torch.Generator().manual_seed(4)).tolist()
+    want, margin = reference(c, weights, toks)
+    d = Driver(folder, dtype, pages=180, page_size=4, max_step_tokens=64)
+    warm = {"w0": toks[:37], "w1": toks[:90]}
+    d.step([("w0", 37), ("w1", 90)], warm)
+    d.end("w0")
+    schedule = [[("a", 330)], [("a", 64)], [("a", 15)], [("a", 2)]] + [[("a", 1)]] * 9 + [[("a", 90)], [("a", 90)]]
+    got = d.run(schedule, {"a": toks})["a"]
+    d.end("w1")
+    err = row_error(got, want)
+    if dtype == "float32":
+        assert err.max() < 1e-3, (int(err.argmax()), float(err.max()))
+    else:
+        behind = np.cumsum(margin < CLOSE) > 0
+        assert np.median(err) < (5 if behind.mean() > 0.5 else 1) * BAR[dtype], float(np.median(err))
+    d.close()
+
+
+def test_a_state_that_remembers_its_first_tokens(device, tmp_path):
+    """One mLSTM layer that forgets nothing (a large bias under the forget gate's cap): the logits at the end depend on
+    the first tokens. Two prompts that differ in their first three tokens only must differ at token 200 and later, and
+    each must match the plain implementation whether it ran whole, or in portions and single tokens."""
+    c = config([dict(mlstm(2, 64, 48, 20.0), mlp=dense(64))], width=64, vocab=50)
+    weights = make_weights(c, seed=4)
+    weights["l0.mix.f.b"] = torch.full((2,), 18.0).to(torch.bfloat16)
+    weights["l0.mix.i.b"] = torch.full((2,), -1.0).to(torch.bfloat16)
+    weights["l0.mix.i"] = weights["l0.mix.i"] * 0.1
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(9)
+    base = torch.randint(0, 50, (260,), generator=g).tolist()
+    other = [(t + 7) % 50 for t in base[:3]] + base[3:]
+    tokens = {"a": base, "b": other}
+    want = {k: plain.forward(c, double(weights), v).numpy() for k, v in tokens.items()}
+    assert row_error(want["a"][200:], want["b"][200:]).min() > 1e-3
+    d = Driver(folder, "float32", pages=40, page_size=16, max_requests=2)
+    got = d.run([[("a", 260)], [("b", 100)], [("b", 2)]] + [[("b", 1)]] * 17 + [[("b", 141)]], tokens)
+    for k in tokens:
+        assert row_error(got[k], want[k]).max() < BAR["float32"], k
+    d.close()
+
+
+def random_config(seed):
+    """A configuration nobody chose: one to six layers of the three kinds in any order, any feed-forward, sizes of every
+    parity, layers that run with an earlier layer's weights."""
+    rng = random.Random(seed)
+    layers = []
+    for _ in range(rng.randint(1, 6)):
+        own = [i for i, lay in enumerate(layers) if lay.get("weights_of") is None]
+        if own and rng.random() < 0.2:
+            j = rng.choice(own)
+            layers.append(same_as(layers[j], j))
+            continue
+        kind = rng.choice(["dense", "moe", "moe", None])
+        if kind == "dense":
+            mlp = dense(rng.choice([24, 40, 100, 136]))
+        elif kind == "moe":
+            experts = rng.choice([1, 2, 6, 9, 33])
+            mlp = moe(experts, rng.randint(1, min(experts, 4)), rng.choice([8, 20, 48, 70]), rng.choice([None, 8, 24, 50]))
+        else:
+            mlp = None
+        which = rng.choice(["attention", "latent", "mlstm"])
+        if which == "attention":
+            G = rng.choice([1, 2, 3])
+            H = G * rng.choice([1, 2, 4])
+            D = rng.choice([8, 12, 34, 64, 80])
+            layers.append(attention(H, G, D, rng.choice([d for d in (2, 4, 8, 12, 34, 64, 80) if d <= D]), rng.uniform(0.05, 0.5),
+                                    rng.randint(1, 5), rng.choice([1, 3, 8, 17, 40, 200]), rng.choice([0, 1, 4, 16, 19]),
+                                    rng.choice([50.0, 1e4, 1e6]), mlp))
+        elif which == "latent":
+            R = rng.choice([2, 8, 16, 24])
+            layers.append(latent(rng.choice([1, 2, 3, 5]), rng.choice([8, 12, 32, 50]), R, rng.choice([8, 20, 64]),
+                                 rng.choice([16, 40, 100, 128]), rng.uniform(0.05, 0.4), rng.choice([50.0, 1e4, 1e6]),
+                                 rng.choice([r for r in (2, 8, 16, 24) if r <= R]), mlp))
+        else:
+            layers.append(mlstm(rng.choice([1, 2, 3, 4]), rng.choice([4, 9, 16, 50, 96, 130]), rng.choice([3, 8, 20, 64, 100]),
+                                rng.choice([2.0, 8.0, 15.0]), mlp))
+    return config(layers, width=rng.choice([40, 56, 100, 136, 192]), vocab=rng.randint(30, 400), mult=rng.choice([1.0, 0.3, 0.5]),
+                  softcap=rng.choice([None, 5.0, 30.0]), eps=rng.choice([1e-6, 1e-5, 1e-3]))
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_configurations_drawn_at_random(device, tmp_path, seed):
+    """Whole prompts in one batch, then a prompt in portions with its last tokens one by one beside another request, in
+    both precisions, for sizes nobody chose."""
+    c = random_config(seed)
+    weights = make_weights(c, seed=100 + seed)
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(seed)
+    tokens = {"a": torch.randint(0, c["vocab"], (83,), generator=g).tolist(), "b": torch.randint(0, c["vocab"], (21,), generator=g).tolist()}
+    want = {k: reference(c, weights, v) for k, v in tokens.items()}
+    for dtype in ("float32", "bfloat16"):
+        d = Driver(folder, dtype, pages=40, page_size=4, max_requests=2)
+        whole = d.run([[("a", 83), ("b", 21)]], tokens)
+        cut = d.run([[("a", 30)], [("a", 17), ("b", 2)], [("a", 2), ("b", 1)], [("a", 24), ("b", 9)]] + [[("a", 1), ("b", 1)]] * 10, tokens)
+        for got in (whole, cut):
+            for k in tokens:
+                check_rows(row_error(got[k], want[k][0]), dtype, (seed, c["width"], k), want[k][1])
+        d.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompt_in_one_step(device, tmp_path, dtype):
+    """1,300 tokens: 1,100 in one step (the mLSTM over many chunks, prompt attention over many tiles, experts with
+    hundreds of rows each), then a portion of 150 behind them and single tokens, beside a second, short request."""
+    c = CONFIGS["odd"]
+    weights = make_weights(c, seed=17)
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(6)
+    tokens = {"a": torch.randint(0, c["vocab"], (1300,), generator=g).tolist(), "b": torch.randint(0, c["vocab"], (40,), generator=g).tolist()}
+    want = {k: reference(c, weights, v) for k, v in tokens.items()}
+    d = Driver(folder, dtype, pages=100, page_size=16, max_requests=2)
+    got = d.run([[("a", 1100), ("b", 3)], [("a", 150), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 36 + [[("a", 14)]], tokens)
+    for k in tokens:
+        check_rows(row_error(got[k], want[k][0]), dtype, k, want[k][1])
+    d.close()
+
+
+def test_long_decoding_from_graphs(device, tmp_path):
+    """400 tokens decoded one by one from graphs after a short prompt, two requests side by side: the window passes
+    over decoded tokens, its pages come back, the kept first ones stay."""
+    c = CONFIGS["odd"]
+    weights = make_weights(c, seed=11)
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(3)
+    tokens = {"a": torch.randint(0, c["vocab"], (420,), generator=g).tolist(),
+              "b": torch.randint(0, c["vocab"], (409,), generator=g).tolist()}
+    want = {k: reference(c, weights, v) for k, v in tokens.items()}
+    d = Driver(folder, "float32", pages=70, page_size=16)
+    got = d.run([[("a", 20), ("b", 9)]] + [[("a", 1), ("b", 1)] for _ in range(400)], tokens)
+    for k in tokens:
+        check_rows(row_error(got[k], want[k][0]), "float32", k, want[k][1])
+    assert d.stepper.graph_replays > 300
+    d.close()
+
+
+@pytest.mark.parametrize("name", ["odd", "wide"])
+def test_greedy_generation_through_the_scheduler(device, tmp_path, name):
+    """`engine_for(...).generate`: the package's entry point, scheduler, sampler and lookahead. Every generated
+    token must be the plain implementation's best token for the text so far (checked where its lead is clear)."""
+    from tessweave_engine_amd.cli import engine_for
+    c = CONFIGS[name]
+    weights = make_weights(c, seed=21)
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(8)
+    prompts = [torch.randint(0, c["vocab"], (n,), generator=g).tolist() for n in (5, 23, 1, 40, 12, 30)]
+    engine = engine_for(folder, dtype="float32", max_context=128, kv_blocks=60, block_size=8, max_active=3,
+                        prefill_chunk=16, no_prefix_cache=False)
+    try:
+        outputs = engine.generate(prompts, max_tokens=24, temperature=0.0)
+    finally:
+        engine.close()
+    clear = 0
+    for prompt, out in zip(prompts, outputs):
+        assert len(out) == 24
+        logits = plain.forward(c, double(weights), prompt + out)[len(prompt) - 1:-1]
+        top = logits.topk(2, -1)
+        for t, token in enumerate(out):
+            if top.values[t, 0] - top.values[t, 1] > 1e-3:
+                assert token == int(top.indices[t, 0]), (t, token)
+                clear += 1
+    assert clear > 100
