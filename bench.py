@@ -19,7 +19,7 @@ as the weights; `prefill_32k_prompts`: tokens a second over those prompts, which
 go through in portions of 2,048); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
 (`gen512_b*`, decoded tokens a second over the generated part).
 
-Other sizes of the architecture: --shape 14b|32b. --design kanavik|dinutar|rufusun measures that
+Other sizes of the architecture: --shape 14b|32b. --design kanavik|dinutar|rufusun|tadalorn measures that
 design's prefill and decode at a few layer sizes, each beside the Qwen2 decoder at equal
 width, heads, feed-forward and depth (one JSON line a size). --serve measures continuous
 batching under Poisson arrivals instead (prompts of 128..4,096 tokens, 256
@@ -89,7 +89,7 @@ def parse():
                    help="with --serve: the largest prompt portion in one step (larger: more prompt tokens a second and "
                         "a shorter time to the first token, longer steps for the requests that are decoding)")
     p.add_argument("--rate", type=float, default=16.0, help="mean arrivals a second (0: all at once)")
-    p.add_argument("--design", default="", choices=["", "kanavik", "dinutar", "rufusun"],
+    p.add_argument("--design", default="", choices=["", "kanavik", "dinutar", "rufusun", "tadalorn"],
                    help="instead: prefill and decode throughput of another design at a few layer sizes (--design-sizes), "
                         "each beside the Qwen2 decoder at equal width, heads, feed-forward and depth; one JSON line a size")
     p.add_argument("--design-sizes", default="1b,3b,7b", help="which of the design's sizes to run, comma separated")
@@ -168,6 +168,33 @@ def rufusun_config(size, layers, context):
             "layers": out}
 
 
+# The Tadalorn design at those widths: layers in the order latent attention, mLSTM, windowed attention, latent attention,
+# the first with a dense feed-forward and the others with routed experts (16 experts of a quarter of the dense inner size,
+# two a token, beside a shared expert of that size, as in the Rufusun run, which is measured beside it). Latent attention:
+# the size's heads, 64 unrotated + 64 rotated query/key elements a head, values of the head size, a latent of 192. mLSTM:
+# the size's heads, keys and values of the head size. Windowed attention: the size's heads, key heads and window, four kept
+# first tokens, convolutions of four taps, rotation over half of a head.
+def tadalorn_config(size, layers, context):
+    width, heads, kv_heads, dim, ff, window = DESIGN_SIZES[size]
+    dense = {"kind": "dense", "ff": ff}
+    routed = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4}}
+    latent = {"heads": heads, "dim": dim - 64, "rot_dim": 64, "vdim": dim, "kv_rank": 192, "scale": dim ** -0.5,
+              "rot": {"base": 50000.0, "dims": 64}}
+    out = []
+    for i in range(layers):
+        mlp = routed if i % 4 else dense
+        if i % 4 in (0, 3):
+            out.append({"type": "latent_attention", "mixer": latent, "mlp": mlp})
+        elif i % 4 == 1:
+            out.append({"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": dim, "gate_cap": 15.0}, "mlp": mlp})
+        else:
+            out.append({"type": "attention", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "conv": 4,
+                                  "mask": {"size": window, "keep_first": 4}, "rot": {"base": 1e6, "dims": dim // 2}}})
+    return {"architecture": "Tadalorn", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "logit_softcap": 30.0, "layers": out}
+
+
 def qwen2_config_like(size, layers, context):
     width, heads, kv_heads, dim, ff, _ = DESIGN_SIZES[size]
     return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
@@ -188,9 +215,12 @@ def design_run(args, torch):
                 "sizes": dict(zip(("width", "heads", "kv_heads", "head_dim", "ff", "window"), DESIGN_SIZES[size])),
                 "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens,
                 "data": "synthetic: uniform-random token ids, random weights"}
-        make = {"kanavik": kanavik_config, "dinutar": dinutar_config, "rufusun": rufusun_config}[args.design]
+        make = {"kanavik": kanavik_config, "dinutar": dinutar_config, "rufusun": rufusun_config,
+                "tadalorn": tadalorn_config}[args.design]
         models = [(args.design, make(size, args.design_layers, args.context))]
         if not args.design_only:
+            if args.design == "tadalorn":          # the closest design of the engine (experts, a recurrence, attention)
+                models.append(("rufusun", rufusun_config(size, args.design_layers, args.context)))
             models.append(("qwen2", qwen2_config_like(size, args.design_layers, args.context)))
         for name, cfg in models:
             model = random_model(config_from_dict(cfg), args.seed, dtype=args.dtype, device="cuda:0")

@@ -70,6 +70,8 @@ struct AttnArgs {
   int tile_rows;          // rows of such a tile: 128, or 64 when there would be too few workgroups
   int kv_chunk, max_chunks;  // prefill (bfloat16 kernel): keys per workgroup (a multiple of 32) and the most
                              // chunks a tile can have; max_chunks == 1: a tile's keys are never split
+  const float* sink;         // prefill only. [q_heads] or null: exp(sink_h) more in head h's denominator (a score of its
+                             // own, not scaled, with no key and no value)
 };
 
 // Per-wave online-softmax state for one 16-row tile. Lane (r, g) belongs to row r.
@@ -610,6 +612,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
   const int t_row = row_ok ? first_pos + tok : -1;
   RowTile<T, DTMAX> tile;
   tile.init(row_ok ? (const T*)a.q + (size_t)(token0 + tok) * a.ldq + (size_t)head * D : nullptr, D, g);
+  if (a.sink && row_ok) {                              // the sink: as a key of score sink_h seen first, with a value of zeros
+    tile.m = a.sink[head];
+    tile.l = 1.f;
+  }
 
   const int t_min = first_pos + row0 / G;
   const int t_max = first_pos + min(rows - 1, row0 + 15) / G;
@@ -1308,6 +1314,11 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   run_to(blk_end, step_by_step);                             // (blk_end > blk_begin always)
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) l[rt] = tw_rows_sum(l[rt]) + l_mma[rt][0];   // (the running maximum, and so every rescaling, was the row's: the same for the four)
+  if (a.sink && n_chunks == 1) {                             // (split tiles: the merge adds it, once)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+      if (row_ok[rt]) l[rt] += __builtin_amdgcn_exp2f(fmaf(a.sink[head[rt]], 1.44269504088896340736f, -m_use[rt]));
+  }
 
   if (n_chunks > 1) {
 #pragma unroll
@@ -1380,6 +1391,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnArgs a) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) o[e] += x[e] * w;
     }
+    if (a.sink) l_all += __builtin_amdgcn_exp2f(fmaf(a.sink[head], 1.44269504088896340736f, -m_use));
     const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
     bf16_t packed[4];
 #pragma unroll
@@ -1564,6 +1576,7 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
   a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = splits;
+  a.sink = nullptr;
   TW_REQUIRE(softcap >= 0.f);
   a.softcap = softcap;
   a.part_o = nullptr; a.part_ml = nullptr;
@@ -1613,8 +1626,9 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
                                const int* kv_len, int seq0, int n_seqs, int max_q_len, void* out,
                                long ldo, float* workspace, long workspace_floats, int n_tokens, int max_chunks,
                                int kv_chunk, int tile_rows, int q_heads, int kv_heads, int head_dim, int page_size,
-                               int window, float scale, float softcap, int generic, hipStream_t stream) {
+                               int window, float scale, float softcap, int generic, const float* sink, hipStream_t stream) {
   AttnArgs a;
+  a.sink = sink;
   TW_REQUIRE(tile_rows == 0 || tile_rows == 64 || tile_rows == 128);
   a.tile_rows = tile_rows;
   a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;

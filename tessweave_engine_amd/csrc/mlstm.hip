@@ -34,6 +34,7 @@ struct MlstmArgs {
   float* out; long ld_out;           // [rows][H E]
   int H, D, E, Dp, Ep;
   float q_scale, cap;
+  int gates_ready;                   // the rows hold i and f already (mlstm_gates_kernel ran), not the gates' raw values
 };
 
 __device__ __forceinline__ float ml_logsigmoid(float z) { return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z)); }
@@ -107,10 +108,12 @@ __global__ __launch_bounds__(256) void mlstm_walk_kernel(MlstmArgs a) {
 }
 
 // grid (ceil(Ep / 64), H, n_seqs), 256 threads; dynamic LDS (ml_chunk_lds_floats).
+// A chunk's rows are held twice in LDS: while chunk c is worked on, the rows of chunk c + 1 are on their way from memory
+// into registers and go to the other copy at the top of the next iteration, so an iteration has two barriers and waits
+// for memory only where the arithmetic of a chunk is shorter than a load.
 #define ML_L 16
-static size_t ml_chunk_lds_floats(int Dp) {
-  return (size_t)2 * ML_L * (Dp + 4) + (size_t)ML_L * 68 + 4 * 64 * 4 + Dp + 5 * ML_L;
-}
+static size_t ml_buffer_floats(int Dp) { return (size_t)2 * ML_L * (Dp + 4) + (size_t)ML_L * 68 + 6 * ML_L; }
+static size_t ml_chunk_lds_floats(int Dp) { return 2 * ml_buffer_floats(Dp) + 4 * 64 * 4 + Dp + ML_L; }
 
 template <int DT>      // key tiles of 16 a wave's part of S spans in registers (Dp <= 16 DT)
 __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
@@ -121,17 +124,12 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int Dp = a.Dp, QS = Dp + 4, tiles = Dp / 16;
-  float* Qs = ml_lds;                          // [16][Dp + 4], scaled queries
-  float* Ks = Qs + ML_L * QS;                  // [16][Dp + 4]
-  float* Vs = Ks + ML_L * QS;                  // [16][68]: this workgroup's 64 value columns
-  f32x4* part = (f32x4*)(Vs + ML_L * 68);      // [4 waves][64 lanes]
-  float* n_s = (float*)(part + 4 * 64);        // [Dp]
-  float* u_s = n_s + Dp;                       // [16] i_j - F_j (minus infinity behind the chunk's last token)
-  float* g_s = u_s + ML_L;                     // [16] running maximum, m0 included
-  float* F_s = g_s + ML_L;                     // [16]
-  float* nq_s = F_s + ML_L;                    // [16] n0 . q_t
+  const size_t buffer = (size_t)2 * ML_L * QS + (size_t)ML_L * 68 + 6 * ML_L;
+  f32x4* part = (f32x4*)(ml_lds + 2 * buffer);  // [4 waves][64 lanes]
+  float* n_s = (float*)(part + 4 * 64);         // [Dp]
+  float* nq_s = n_s + Dp;                       // [16] n0 . q_t
   const int slot = a.state_slots[seq], ph = a.phase[seq] & 1;
-  const int v0 = blockIdx.x * 64 + wave * 16;  // this wave's value columns v0 .. v0 + 15
+  const int v0 = blockIdx.x * 64 + wave * 16;   // this wave's value columns v0 .. v0 + 15
   const bool wave_on = v0 < a.Ep;
   float* S = a.S + (((size_t)slot * a.H + head) * a.Ep + v0 + r) * Dp;
   const float* n_in = a.n + (((size_t)slot * 2 + ph) * a.H + head) * Dp;
@@ -143,29 +141,79 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
   for (int d = threadIdx.x; d < Dp; d += 256) n_s[d] = n_in[d];
   float m0 = a.m[((size_t)slot * 2 + ph) * a.H + head];
 
-  for (int c0 = r0; c0 < r1; c0 += ML_L) {
+  // ---- a chunk's rows on their way: groups of four elements, QK groups of q and of k a thread, one of v ------------
+  constexpr int QK = DT / 4;                     // 16 rows x Dp / 4 groups over 256 threads
+  const int groups = Dp / 4;                     // of a row of q or k
+  const bool vec = a.D % 4 == 0 && a.E % 4 == 0 && a.ld % 4 == 0 && a.q_col % 4 == 0 && a.k_col % 4 == 0 && a.v_col % 4 == 0 &&
+                   (uintptr_t)a.proj % 16 == 0;
+  f32x4 q_in[QK], k_in[QK], v_in;
+  float gate_i = 0.f, gate_f = 0.f;
+  auto four = [&](const float* p, int first, int size) -> f32x4 {      // elements first .. first + 3 of a head's `size`
+    f32x4 x = {0.f, 0.f, 0.f, 0.f};
+    if (vec) {
+      if (first < size) x = *reinterpret_cast<const f32x4*>(p + first);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (first + e < size) x[e] = p[first + e];
+    }
+    return x;
+  };
+  auto request = [&](int c0) {
     const int valid = min(ML_L, r1 - c0);
-    // ---- 1: the chunk's rows and gates into LDS ------------------------------------------------------------
-    for (int i = threadIdx.x; i < ML_L * Dp; i += 256) {
-      const int t = i / Dp, d = i - t * Dp;
-      float qv = 0.f, kv = 0.f;
-      if (t < valid && d < a.D) {
+#pragma unroll
+    for (int i = 0; i < QK; ++i) {
+      const int item = threadIdx.x + i * 256;
+      const int t = item / groups, d = (item - t * groups) * 4;
+      q_in[i] = k_in[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (t < valid && item < ML_L * groups) {
         const float* row = a.proj + (size_t)(c0 + t) * a.ld;
-        qv = row[a.q_col + head * a.D + d] * a.q_scale;
-        kv = row[a.k_col + head * a.D + d];
+        q_in[i] = four(row + a.q_col + head * a.D, d, a.D);
+        k_in[i] = four(row + a.k_col + head * a.D, d, a.D);
       }
-      Qs[t * QS + d] = qv;
-      Ks[t * QS + d] = kv;
     }
-    for (int i = threadIdx.x; i < ML_L * 64; i += 256) {
-      const int t = i >> 6, c = i & 63;
-      const int v = blockIdx.x * 64 + c;
-      Vs[t * 68 + c] = (t < valid && v < a.E) ? a.proj[(size_t)(c0 + t) * a.ld + a.v_col + head * a.E + v] : 0.f;
+    {
+      const int t = threadIdx.x >> 4, c = (threadIdx.x & 15) * 4;
+      v_in = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (t < valid) v_in = four(a.proj + (size_t)(c0 + t) * a.ld + a.v_col + head * a.E, blockIdx.x * 64 + c, a.E);
     }
+    if (threadIdx.x < ML_L && threadIdx.x < valid) {
+      const float* row = a.proj + (size_t)(c0 + threadIdx.x) * a.ld;
+      gate_i = row[a.i_col + head];
+      gate_f = row[a.f_col + head];
+    }
+  };
+  request(r0);
+  int cur = 0;
+  for (int c0 = r0; c0 < r1; c0 += ML_L, cur ^= 1) {
+    const int valid = min(ML_L, r1 - c0);
+    float* Qs = ml_lds + cur * buffer;          // [16][Dp + 4], scaled queries
+    float* Ks = Qs + ML_L * QS;                 // [16][Dp + 4]
+    float* Vs = Ks + ML_L * QS;                 // [16][68]: this workgroup's 64 value columns
+    float* u_s = Vs + ML_L * 68;                // [16] i_j - F_j (minus infinity behind the chunk's last token)
+    float* g_s = u_s + ML_L;                    // [16] running maximum, m0 included
+    float* F_s = g_s + ML_L;                    // [16]
+    float* e_s = F_s + ML_L;                    // [16] exp(u_j - g_last): what key j adds to the state after the chunk
+    float* c_s = e_s + ML_L;                    // [16] exp(m0 - g_t): what is left of the state before the chunk at token t
+    float* f_s = c_s + ML_L;                    // [16] exp(-m_t): the floor of token t's denominator
+    // ---- 1: the chunk's rows and gates into LDS -------------------------------------------------------------
+#pragma unroll
+    for (int i = 0; i < QK; ++i) {
+      const int item = threadIdx.x + i * 256;
+      const int t = item / groups, d = (item - t * groups) * 4;
+      if (item < ML_L * groups) {
+        *reinterpret_cast<f32x4*>(Qs + t * QS + d) = q_in[i] * a.q_scale;
+        *reinterpret_cast<f32x4*>(Ks + t * QS + d) = k_in[i];
+      }
+    }
+    *reinterpret_cast<f32x4*>(Vs + (threadIdx.x >> 4) * 68 + (threadIdx.x & 15) * 4) = v_in;
     if (threadIdx.x < ML_L) {
       const int t = threadIdx.x;
       float i_log = 0.f, f_log = 0.f;
-      if (t < valid) ml_gates(a, a.proj + (size_t)(c0 + t) * a.ld, head, i_log, f_log);
+      if (t < valid) {
+        i_log = a.gates_ready ? gate_i : a.cap * tanhf((gate_i + a.i_bias[head]) / a.cap);
+        f_log = a.gates_ready ? gate_f : ml_logsigmoid(a.cap * tanhf((gate_f + a.f_bias[head]) / a.cap));
+      }
       float F = f_log;                            // inclusive running sum over the 16 lanes
 #pragma unroll
       for (int o = 1; o < ML_L; o <<= 1) {
@@ -182,8 +230,13 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
       u_s[t] = u;
       g_s[t] = best;
       F_s[t] = F;
+      const float g_end = __shfl(best, valid - 1, TW_WAVE);
+      e_s[t] = t < valid ? expf(u - g_end) : 0.f;
+      c_s[t] = expf(m0 - best);
+      f_s[t] = expf(-(F + best));
     }
     __syncthreads();
+    if (c0 + ML_L < r1) request(c0 + ML_L);       // the next chunk's rows travel while this one is worked on
     // ---- 2: K Q^T over this wave's share of the key elements; n0 . q_t ------------------------------------
     {
       f32x4 p = {0.f, 0.f, 0.f, 0.f};
@@ -204,7 +257,7 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
     // ---- 3: weights, outputs, the new state -------------------------------------------------------------------
     const int last = valid - 1;
     const float g_last = g_s[last];
-    const float carry = expf(m0 - g_last);        // what is left of the state before the chunk
+    const float carry = c_s[last];                // what is left of the state before the chunk
     if (wave_on) {
       f32x4 w = part[lane] + part[64 + lane] + part[128 + lane] + part[192 + lane];
       const float g_t = g_s[r];
@@ -216,22 +269,26 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
         rows += w[e];
       }
       rows = tw_rows_sum(rows);
-      const float nq = __fmaf_rn(expf(m0 - g_t), nq_s[r], rows);
-      const float den = fmaxf(fabsf(nq), expf(-(F_s[r] + g_t))) + 1e-6f;   // of token r
+      const float nq = __fmaf_rn(c_s[r], nq_s[r], rows);
+      const float den = fmaxf(fabsf(nq), f_s[r]) + 1e-6f;                  // of token r
       // values of keys 4 g .. 4 g + 3, column v0 + r
       f32x4 vf;
 #pragma unroll
       for (int e = 0; e < 4; ++e) vf[e] = Vs[(4 * g + e) * 68 + wave * 16 + r];
-      f32x4 o = {0.f, 0.f, 0.f, 0.f};
+      f32x4 o = {0.f, 0.f, 0.f, 0.f}, o2 = {0.f, 0.f, 0.f, 0.f};          // (two chains of products instead of one)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
+      for (int dt = 0; dt < DT; dt += 2) {
         if (dt < tiles) {
           const f32x4 qf = *reinterpret_cast<const f32x4*>(Qs + r * QS + dt * 16 + 4 * g);
           tw_mma16_k4(o, qf, acc[dt]);            // o[e]: token 4 g + e, column v0 + r
         }
+        if (dt + 1 < tiles) {
+          const f32x4 qf = *reinterpret_cast<const f32x4*>(Qs + r * QS + (dt + 1) * 16 + 4 * g);
+          tw_mma16_k4(o2, qf, acc[dt + 1]);
+        }
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] *= expf(m0 - g_s[4 * g + e]);
+      for (int e = 0; e < 4; ++e) o[e] = (o[e] + o2[e]) * c_s[4 * g + e];
       tw_mma16_k4(o, w, vf);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -243,7 +300,7 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
       // S <- carry S + sum_j exp(u_j - g_last) k_j v_j^T
       float ej[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) ej[e] = (4 * g + e) < valid ? expf(u_s[4 * g + e] - g_last) : 0.f;
+      for (int e = 0; e < 4; ++e) ej[e] = e_s[4 * g + e];
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         if (dt < tiles) {
@@ -258,12 +315,14 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
     }
     for (int d = threadIdx.x; d < Dp; d += 256) {
       float sum = carry * n_s[d];
-      for (int j = 0; j < valid; ++j) sum = __fmaf_rn(expf(u_s[j] - g_last), Ks[j * QS + d], sum);
+      for (int j = 0; j < valid; ++j) sum = __fmaf_rn(e_s[j], Ks[j * QS + d], sum);
       n_s[d] = sum;
     }
     m0 = F_s[last] + g_last;
-    __syncthreads();
+    // (no barrier here: the next iteration writes the other copy of the rows, and what it shares with this one, part, n_s
+    // and nq_s, is written behind its first barrier, which every wave reaches only when it is done here)
   }
+  __syncthreads();
   if (wave_on) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -275,11 +334,22 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
   }
 }
 
+// The two gates of rows first_row .. n - 1, all heads, in place of their raw values: off the chunks' chain of dependent steps.
+__global__ void mlstm_gates_kernel(float* proj, long ld, int i_col, int f_col, const float* __restrict__ i_bias,
+                                   const float* __restrict__ f_bias, float cap, int first_row, int n, int H) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)(n - first_row) * H) return;
+  const int head = (int)(i % H);
+  float* row = proj + (size_t)(first_row + i / H) * ld;
+  row[i_col + head] = cap * tanhf((row[i_col + head] + i_bias[head]) / cap);
+  row[f_col + head] = ml_logsigmoid(cap * tanhf((row[f_col + head] + f_bias[head]) / cap));
+}
+
 // Sequences seq0 .. seq0 + n_seqs - 1. walk != 0: token by token (steps of a few tokens), else in chunks of 16.
-extern "C" int tw_mlstm(const float* proj, long ld, int q_col, int k_col, int v_col, int i_col, int f_col, const float* i_bias,
+extern "C" int tw_mlstm(float* proj, long ld, int q_col, int k_col, int v_col, int i_col, int f_col, const float* i_bias,
                         const float* f_bias, float* S, float* n, float* m, const int* q_start, const int* state_slots,
                         const int* phase, int seq0, int n_seqs, float* out, long ld_out, int H, int D, int E, float q_scale,
-                        float cap, int walk, hipStream_t stream) {
+                        float cap, int walk, int first_row, int n_rows, hipStream_t stream) {
   TW_REQUIRE(proj && i_bias && f_bias && S && n && m && q_start && state_slots && phase && out);
   TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && H > 0 && D > 0 && D <= 256 && E > 0 && cap > 0.f);
   TW_REQUIRE(q_col >= 0 && k_col >= 0 && v_col >= 0 && i_col >= 0 && f_col >= 0);
@@ -289,15 +359,29 @@ extern "C" int tw_mlstm(const float* proj, long ld, int q_col, int k_col, int v_
   const int Dp = (D + 15) / 16 * 16, Ep = (E + 15) / 16 * 16;
   TW_REQUIRE((uintptr_t)S % 16 == 0);
   MlstmArgs a{proj, ld, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, S, n, m, q_start, state_slots, phase, seq0,
-              out, ld_out, H, D, E, Dp, Ep, q_scale, cap};
+              out, ld_out, H, D, E, Dp, Ep, q_scale, cap, 0};
   if (walk) {
     mlstm_walk_kernel<<<dim3(Ep / 16, H, n_seqs), 256, 0, stream>>>(a);
     return TW_LAUNCH_RESULT();
   }
+  // first_row >= 0: the launch's sequences own rows first_row .. n_rows - 1 of proj, whose gates are formed first, in place
+  if (first_row >= 0 && n_rows > first_row) {
+    const long items = (long)(n_rows - first_row) * H;
+    mlstm_gates_kernel<<<tw_div_up(items, 256), 256, 0, stream>>>(proj, ld, i_col, f_col, i_bias, f_bias, cap, first_row, n_rows, H);
+    a.gates_ready = 1;
+  }
   const dim3 grid(tw_div_up(Ep, 64), H, n_seqs);
   const size_t lds = ml_chunk_lds_floats(Dp) * sizeof(float);
-  if (Dp <= 64) mlstm_chunk_kernel<4><<<grid, 256, lds, stream>>>(a);
-  else if (Dp <= 128) mlstm_chunk_kernel<8><<<grid, 256, lds, stream>>>(a);
-  else mlstm_chunk_kernel<16><<<grid, 256, lds, stream>>>(a);
+  if (Dp <= 64) {
+    mlstm_chunk_kernel<4><<<grid, 256, lds, stream>>>(a);
+  } else if (Dp <= 128) {
+    mlstm_chunk_kernel<8><<<grid, 256, lds, stream>>>(a);
+  } else {
+    if (lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void*)mlstm_chunk_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+    }
+    mlstm_chunk_kernel<16><<<grid, 256, lds, stream>>>(a);
+  }
   return TW_LAUNCH_RESULT();
 }

@@ -36,7 +36,7 @@ _SIGNATURES = {
     "tw_attn_decode": (I, [I, P, L, P, P, P, I, P, P, I, I, P, L, P, L, I, I, I, I, I, F, F, I, I, P]),
     "tw_attn_prefill_split": (I, [I, I, I, I, I, I, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "tw_attn_prefill_workspace_floats": (L, [I, I, I, I]),
-    "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P]),
+    "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P, P]),
     "tw_add_table_rows": (I, [I, P, P, P, I, I, I, P, P]),
     "tw_causal_conv": (I, [I, I, P, L, P, F, P, P, F, P, P, P, P, P, P, L, P, L, I, I, I, I, P, I, P]),
     "tw_gated_recurrence_workspace_floats": (L, [I, I, I]),
@@ -77,7 +77,7 @@ _SIGNATURES = {
     "tw_sigmoid_gate": (I, [I, P, L, P, L, I, I, I, P]),
     "tw_softcap_values": (I, [P, L, F, P]),
     "tw_qk_finish": (I, [I, P, L, I, I, P, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, I, F, P]),
-    "tw_mlstm": (I, [P, L, I, I, I, I, I, P, P, P, P, P, P, P, P, I, I, P, L, I, I, I, F, F, I, P]),
+    "tw_mlstm": (I, [P, L, I, I, I, I, I, P, P, P, P, P, P, P, P, I, I, P, L, I, I, I, F, F, I, I, I, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),
     "tw_sample_rows": (I, [P, L, I, I, P, P, P, P, P, L, P]),

@@ -433,8 +433,11 @@ def attn_prefill_workspace_floats(n_tokens, q_heads, head_dim, max_chunks):
 
 
 def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_q_len, out, q_heads,
-                 kv_heads, head_dim, scale, window=0, generic=False, split=None, workspace=None, softcap=0.0):
+                 kv_heads, head_dim, scale, window=0, generic=False, split=None, workspace=None, softcap=0.0, sink=None):
     """Attention of sequences seq0..seq0+n_seqs-1 with up to max_q_len query tokens each.
+
+    sink float32 [q_heads]: exp(sink_h) more in head h's softmax denominator (a score of its own, not scaled, with
+    no key and no value).
 
     split = (max_chunks, kv_chunk[, tile_rows]) from attn_prefill_split with a float32 workspace of
     attn_prefill_workspace_floats(rows of q, ...) lets the fast bfloat16 kernel cut long key ranges
@@ -442,6 +445,7 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
     """
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
+    _need(sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == q_heads), "sink must be float32 [q_heads]")
     max_chunks, kv_chunk, ws_ptr, ws_floats = 1, 0, None, 0
     tile_rows = int(split[2]) if split is not None and len(split) > 2 else 0
     if split is not None and split[0] > 1:
@@ -454,7 +458,7 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
                                     seq0, n_seqs, int(max_q_len), _dev(out), ldo, ws_ptr, ws_floats, q.shape[0],
                                     max_chunks, kv_chunk, tile_rows, q_heads, kv_heads, head_dim,
                                     keys.shape[2], int(window or 0), float(scale), float(softcap or 0.0),
-                                    1 if generic else 0, _stream()), "attn_prefill")
+                                    1 if generic else 0, _dev(sink) if sink is not None else None, _stream()), "attn_prefill")
     return out
 
 
@@ -1281,12 +1285,14 @@ MLSTM_WALK_TOKENS = 4          # sequences with up to this many tokens in a step
 
 
 def mlstm(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, S, n_state, m_state, q_start, state_slots, phase, seq0,
-          n_seqs, out, heads, dim, value_dim, q_scale, cap, walk):
+          n_seqs, out, heads, dim, value_dim, q_scale, cap, walk, first_row=None):
     """The mLSTM's matrix memory over sequences seq0 .. seq0 + n_seqs - 1 of a step. proj float32 rows with q, k
     (heads * dim each), v (heads * value_dim) and the two gates' raw values (heads each) at the given columns; i_bias,
     f_bias float32 [heads]. S float32 [requests, heads, value_dev, dim_dev], n_state [requests, 2, heads, dim_dev], m_state
     [requests, 2, heads] (copy phase[s] is read, the other written). out float32 [rows, heads * value_dim]: S^T q over its
-    denominator. walk: token by token (steps of a few tokens a sequence), else chunks of 16 on the matrix unit."""
+    denominator. walk: token by token (steps of a few tokens a sequence), else chunks of 16 on the matrix unit; then
+    first_row, if given, says that the launch's sequences own the rows from there to proj's last: their gates are formed
+    first by a kernel of their own, IN PLACE of the raw values in proj."""
     n, width, ld = _rows(proj, "proj")
     no, wo, ld_out = _rows(out, "out")
     dim_dev, value_dev = (dim + 15) // 16 * 16, (value_dim + 15) // 16 * 16
@@ -1306,5 +1312,5 @@ def mlstm(proj, q_col, k_col, v_col, i_col, f_col, i_bias, f_bias, S, n_state, m
                              _dev(S), _dev(n_state), _dev(m_state), _dev(q_start, torch.int32, "q_start"),
                              _dev(state_slots, torch.int32, "state_slots"), _dev(phase, torch.int32, "phase"), int(seq0),
                              int(n_seqs), _dev(out), ld_out, int(heads), int(dim), int(value_dim), float(q_scale), float(cap),
-                             1 if walk else 0, _stream()), "mlstm")
+                             1 if walk else 0, -1 if (walk or first_row is None) else int(first_row), n, _stream()), "mlstm")
     return out

@@ -95,8 +95,8 @@ def _check_mixer(kind, m, i):
         for key in ("rot_dim", "kv_rank"):
             _positive(_need(m, key, where), f"layer {i}: {key}")
         _positive_float(_need(m, "scale", where), f"layer {i}: scale")
-        if max(m["dim"] + m["rot_dim"], m["vdim"]) > 256 or m["heads"] > 32:
-            raise ConfigError(f"layer {i}: the attention kernels take heads (dim + rot_dim, vdim) up to 256 and up to 32 heads")
+        if max(m["dim"] + m["rot_dim"], m["vdim"]) > 256:
+            raise ConfigError(f"layer {i}: the attention kernels take heads (dim + rot_dim, vdim) up to 256")
         _check_rot(m, i, m["rot_dim"])
     else:
         if m["dim"] > 256:

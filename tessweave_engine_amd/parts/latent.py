@@ -16,7 +16,7 @@ layer (`LayerRun(writes_cache=False)`): it then has no down-projection of its ow
 layer's c and kr with its own queries and its own W_uk, W_uv.
 
 Options: a learned sink per head (`sink_name`: exp(sink_a) more in head a's denominator, with no key and no value, not
-scaled; prompt portions then run the attention kernel that takes sinks), an output gate (`gate_name`: the heads'
+scaled), an output gate (`gate_name`: the heads'
 results times sigmoid(W_g h) before the output product), and a rotary encoding that pairs neighbouring elements: the
 rotated rows of W_q and of the down-projection are then reordered once, when the weights are bound, into the order
 that pairs element j with j + rot/2 (both sides of every score alike, so no score changes).
@@ -50,8 +50,6 @@ class LatentAttention(Mixer):
             raise ValueError("the rotated part needs a rotary encoding of at most rot_dim elements")
         self.sink_name = prefix + sink_name if sink_name else None
         self.gate_name = prefix + gate_name if gate_name else None
-        if self.sink_name and self.heads > 32:
-            raise ValueError("the attention kernel that takes sinks holds up to 32 heads")
         self.sink = None
         # sizes on the device: tails of zeros, which add nothing to a product
         self.dim_dev = _round_up(dim, 8)
@@ -192,21 +190,12 @@ class LatentAttention(Mixer):
             own_keys = ctx.workspace.get("latent.keys", (own_pages, H, page, hd), ctx.dtype)
             own_values = ctx.workspace.get("latent.values", (own_pages, H, hd, page), ctx.dtype)
             ops.latent_expand_store(up, rows, Lp, own_keys, own_values, H, self.dim, self.rot_dim, self.value_dim)
-            if self.sink is not None:
-                splits = ops.attn_mixed_prefill_splits(n - nd, portions, ctx.max_kv_len)
-                ws = None
-                if splits > 1:
-                    floats = ops.attn_mixed_workspace_floats(portions, longest_portion, H, hd, splits)
-                    ws = ctx.workspace.get("latent.sink.split", (floats,), torch.float32)
-                ops.attn_mixed(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd, portions, longest_portion,
-                               out, H, H, self.scale, sink=self.sink, splits=splits, workspace=ws)
-            else:
-                split = ops.attn_prefill_split(portions, H, H, longest_portion, ctx.max_kv_len)
-                ws = None
-                if split[0] > 1:
-                    ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, hd, split[0]),), torch.float32)
-                ops.attn_prefill(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd,
-                                 portions, longest_portion, out, H, H, hd, self.scale, split=split, workspace=ws)
+            split = ops.attn_prefill_split(portions, H, H, longest_portion, ctx.max_kv_len)
+            ws = None
+            if split[0] > 1:
+                ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, hd, split[0]),), torch.float32)
+            ops.attn_prefill(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd,
+                             portions, longest_portion, out, H, H, hd, self.scale, split=split, workspace=ws, sink=self.sink)
         if self.gate_name:
             ops.sigmoid_gate(out, proj[:, self.g_col:self.g_col + H * hd])
         if ctx.defer_sums and self.o.deferrable(n):

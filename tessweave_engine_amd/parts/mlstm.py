@@ -95,7 +95,8 @@ class MatrixLSTM(Mixer):
             if ctx.n_decode:
                 ops.mlstm(*common, 0, ctx.n_decode, *tail, walk=True)
             if portions:
-                ops.mlstm(*common, ctx.n_decode, portions, *tail, walk=False)
+                # (one-token sequences own the first rows of a step: the portions' rows are the rest)
+                ops.mlstm(*common, ctx.n_decode, portions, *tail, walk=False, first_row=ctx.n_decode)
         act = ctx.scratch("mlstm.act", (n, H * E))
         ops.head_norm_gate(result, proj[:, col["g"]:col["g"] + H * E], self.norm_weight, act, H, E, self.eps,
                            gate_activation="sigmoid")

@@ -264,7 +264,7 @@ def mlstm_plain_heads(proj, H, D, E, i_b, f_b, cap):
     return torch.stack([plain.mlstm_steps(q[:, a], k[:, a], v[:, a], i_log[:, a], f_log[:, a]) for a in range(H)], 1).reshape(T, H * E)
 
 
-@pytest.mark.parametrize("walk", [True, False], ids=["walked", "chunks"])
+@pytest.mark.parametrize("walk", [True, False, None], ids=["walked", "chunks", "chunks_gates_first"])
 @pytest.mark.parametrize("H,D,E", [(3, 20, 24), (1, 13, 10), (2, 128, 64), (4, 32, 80), (2, 256, 16), (1, 64, 200)])
 def test_mlstm_over_cut_sequences_in_reused_slots(device, H, D, E, walk):
     """Three sequences cut differently (one whole, one in portions of 1, 2, 5 and 33 tokens, one token by token), their
@@ -303,7 +303,7 @@ def test_mlstm_over_cut_sequences_in_reused_slots(device, H, D, E, walk):
         proj = torch.cat(rows).contiguous()
         out = torch.full((proj.shape[0], H * E), float("nan"), device=device)
         ops.mlstm(proj, 0, H * D, 2 * H * D, width - 2 * H, width - H, i_b, f_b, S, n_st, m_st, ints(q_start, device), ints(sl, device),
-                  ints(ph, device), 0, len(sl), out, H, D, E, D ** -0.5, cap, walk)
+                  ints(ph, device), 0, len(sl), out, H, D, E, D ** -0.5, cap, bool(walk), first_row=0 if walk is None else None)
         for j, (s, lo, n) in enumerate(who):
             outs[s][lo:lo + n] = out[q_start[j]:q_start[j + 1]]
     for s in range(3):
@@ -506,9 +506,9 @@ def test_ways_of_cutting_agree(model):
 def test_sharp_attention_over_a_long_prompt(device, tmp_path, dtype, name):
     """Scores eight times as large: every softmax sits on one or two keys, wherever they lie among hundreds (far back,
     at a page's edge, a kept first token, the window's last). 600 tokens: 330 in one step, then portions of 64, 15, 2
-    and single tokens, on pages of four tokens handed out in an order of their own. float32 rows must agree to 1e-3,
-    where a key that is lost or seen wrongly moves a row by a tenth and more; in bfloat16 the typical row must stay
-    within the bar."""
+    and single tokens, on pages of four tokens handed out in an order of their own. float32 rows must agree to 1e-3 (plus
+    what float32 arithmetic moves the row by in the plain implementation), where a key that is lost or seen wrongly moves
+    a row by a tenth and more; in bfloat16 the typical row must stay within the bar."""
     c = CONFIGS[name]
     weights = make_weights(c, seed=13, sharp=8.0 if dtype == "float32" else 2.0)
     folder = write_folder(tmp_path, c, weights)
@@ -523,7 +523,8 @@ def test_sharp_attention_over_a_long_prompt(device, tmp_path, dtype, name):
     d.end("w1")
     err = row_error(got, want)
     if dtype == "float32":
-        assert err.max() < 1e-3, (int(err.argmax()), float(err.max()))
+        allowed = 1e-3 + 3.0 * margin.float32
+        assert (err < allowed).all(), (int((err / allowed).argmax()), float(err.max()))
     else:
         behind = np.cumsum(margin < CLOSE) > 0
         assert np.median(err) < (5 if behind.mean() > 0.5 else 1) * BAR[dtype], float(np.median(err))
