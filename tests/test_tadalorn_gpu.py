@@ -123,7 +123,9 @@ def paged(k, v, page, order_seed, device, dtype, dim_dev):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,G,D,rot,window,keep,page", [(4, 2, 24, 16, 9, 3, 4), (8, 8, 32, 32, 64, 0, 16), (4, 1, 64, 32, 5, 20, 8),
-                                                        (2, 2, 16, 0, 33, 1, 16), (6, 3, 40, 8, 16, 16, 4), (3, 3, 128, 128, 40, 4, 16)])
+                                                        (2, 2, 16, 0, 33, 1, 16), (6, 3, 40, 8, 16, 16, 4), (3, 3, 128, 128, 40, 4, 16),
+                                                        (16, 4, 32, 16, 24, 2, 8), (12, 12, 16, 8, 10, 17, 4), (24, 8, 16, 16, 31, 5, 16),
+                                                        (32, 4, 64, 32, 48, 1, 16)])
 def test_window_with_kept_first_keys_and_a_sink_made_sharp(device, dtype, H, G, D, rot, window, keep, page):
     """Whole-row norms, rotation of pairs, cache write and the attention kernel, against the plain softmax over the
     plain mask. Every query row is made to point at ONE key with a large score: the key just inside its window, the one
@@ -361,6 +363,8 @@ ONE_LAYER = {
     "attention_no_keep_one_tap": attention(2, 2, 16, 16, 0.25, 1, 7, 0),
     "latent": latent(3, 24, 8, 40, 48, 0.2, base=500.0),
     "latent_large": latent(2, 40, 24, 96, 250, 0.1),             # a latent too large for the one-head kernel
+    "latent_many_heads": latent(20, 8, 8, 12, 40, 0.3),          # more heads than one tile of the one-token kernel holds
+    "attention_many_heads": attention(24, 6, 16, 8, 0.3, 2, 13, 3),
     "mlstm": mlstm(3, 20, 24, 8.0),
     "dense": dict(mlstm(1, 16, 16, 4.0), mlp=dense(72)),
     "experts": dict(mlstm(1, 16, 16, 4.0), mlp=moe(7, 3, 40, shared=24)),
