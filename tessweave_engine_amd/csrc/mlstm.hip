@@ -37,6 +37,23 @@ struct MlstmArgs {
   int gates_ready;                   // the rows hold i and f already (mlstm_gates_kernel ran), not the gates' raw values
 };
 
+// Inside a row of 16 lanes (DPP): the value of the lane N below (FILL where there is none), and the sum over the row.
+template <int N>
+__device__ __forceinline__ float ml_row_below(float v, float fill) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x110 + N, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ float ml_row_turned(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float ml_row_sum(float v) {      // every lane of the row gets it
+  v += ml_row_turned<0x128>(v);                             // the row rotated by 8 lanes, then by 4, 2, 1
+  v += ml_row_turned<0x124>(v);
+  v += ml_row_turned<0x122>(v);
+  v += ml_row_turned<0x121>(v);
+  return v;
+}
+
 __device__ __forceinline__ float ml_logsigmoid(float z) { return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z)); }
 
 __device__ __forceinline__ void ml_gates(const MlstmArgs& a, const float* row, int head, float& i_log, float& f_log) {
@@ -86,11 +103,8 @@ __global__ __launch_bounds__(256) void mlstm_walk_kernel(MlstmArgs a) {
         pn = __fmaf_rn(nn[j], qd, pn);
       }
     }
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) {
-      po += __shfl_xor(po, o, TW_WAVE);
-      pn += __shfl_xor(pn, o, TW_WAVE);
-    }
+    po = ml_row_sum(po);
+    pn = ml_row_sum(pn);
     if (sl == 0 && v < a.E)
       a.out[(size_t)row_i * a.ld_out + head * a.E + v] = po / (fmaxf(fabsf(pn), expf(-m)) + 1e-6f);
   }
@@ -108,9 +122,9 @@ __global__ __launch_bounds__(256) void mlstm_walk_kernel(MlstmArgs a) {
 }
 
 // grid (ceil(Ep / 64), H, n_seqs), 256 threads; dynamic LDS (ml_chunk_lds_floats).
-// A chunk's rows are held twice in LDS: while chunk c is worked on, the rows of chunk c + 1 are on their way from memory
-// into registers and go to the other copy at the top of the next iteration, so an iteration has two barriers and waits
-// for memory only where the arithmetic of a chunk is shorter than a load.
+// A chunk's rows are held twice in LDS and requested TWO chunks ahead: while chunk c is worked on, the rows of chunks
+// c + 1 and c + 2 are in registers or on their way there from memory (a load takes longer than a chunk's arithmetic), and
+// go to the other copy in LDS at the top of their iteration, so an iteration has two barriers and hardly waits for memory.
 #define ML_L 16
 static size_t ml_buffer_floats(int Dp) { return (size_t)2 * ML_L * (Dp + 4) + (size_t)ML_L * 68 + 6 * ML_L; }
 static size_t ml_chunk_lds_floats(int Dp) { return 2 * ml_buffer_floats(Dp) + 4 * 64 * 4 + Dp + ML_L; }
@@ -146,8 +160,11 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
   const int groups = Dp / 4;                     // of a row of q or k
   const bool vec = a.D % 4 == 0 && a.E % 4 == 0 && a.ld % 4 == 0 && a.q_col % 4 == 0 && a.k_col % 4 == 0 && a.v_col % 4 == 0 &&
                    (uintptr_t)a.proj % 16 == 0;
-  f32x4 q_in[QK], k_in[QK], v_in;
-  float gate_i = 0.f, gate_f = 0.f;
+  struct Rows {
+    f32x4 q[QK], k[QK], v;
+    float gate_i, gate_f;
+  };
+  Rows even, odd;                                // the rows of the chunks with even and with odd numbers
   auto four = [&](const float* p, int first, int size) -> f32x4 {      // elements first .. first + 3 of a head's `size`
     f32x4 x = {0.f, 0.f, 0.f, 0.f};
     if (vec) {
@@ -159,33 +176,34 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
     }
     return x;
   };
-  auto request = [&](int c0) {
+  auto request = [&](int c0, Rows& in) __attribute__((always_inline)) {
     const int valid = min(ML_L, r1 - c0);
 #pragma unroll
     for (int i = 0; i < QK; ++i) {
       const int item = threadIdx.x + i * 256;
       const int t = item / groups, d = (item - t * groups) * 4;
-      q_in[i] = k_in[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      in.q[i] = in.k[i] = f32x4{0.f, 0.f, 0.f, 0.f};
       if (t < valid && item < ML_L * groups) {
         const float* row = a.proj + (size_t)(c0 + t) * a.ld;
-        q_in[i] = four(row + a.q_col + head * a.D, d, a.D);
-        k_in[i] = four(row + a.k_col + head * a.D, d, a.D);
+        in.q[i] = four(row + a.q_col + head * a.D, d, a.D);
+        in.k[i] = four(row + a.k_col + head * a.D, d, a.D);
       }
     }
     {
       const int t = threadIdx.x >> 4, c = (threadIdx.x & 15) * 4;
-      v_in = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (t < valid) v_in = four(a.proj + (size_t)(c0 + t) * a.ld + a.v_col + head * a.E, blockIdx.x * 64 + c, a.E);
+      in.v = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (t < valid) in.v = four(a.proj + (size_t)(c0 + t) * a.ld + a.v_col + head * a.E, blockIdx.x * 64 + c, a.E);
     }
+    in.gate_i = in.gate_f = 0.f;
     if (threadIdx.x < ML_L && threadIdx.x < valid) {
       const float* row = a.proj + (size_t)(c0 + threadIdx.x) * a.ld;
-      gate_i = row[a.i_col + head];
-      gate_f = row[a.f_col + head];
+      in.gate_i = row[a.i_col + head];
+      in.gate_f = row[a.f_col + head];
     }
   };
-  request(r0);
-  int cur = 0;
-  for (int c0 = r0; c0 < r1; c0 += ML_L, cur ^= 1) {
+  request(r0, even);
+  if (r0 + ML_L < r1) request(r0 + ML_L, odd);
+  auto link = [&](int c0, int cur, Rows& in) __attribute__((always_inline)) {
     const int valid = min(ML_L, r1 - c0);
     float* Qs = ml_lds + cur * buffer;          // [16][Dp + 4], scaled queries
     float* Ks = Qs + ML_L * QS;                 // [16][Dp + 4]
@@ -202,31 +220,29 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
       const int item = threadIdx.x + i * 256;
       const int t = item / groups, d = (item - t * groups) * 4;
       if (item < ML_L * groups) {
-        *reinterpret_cast<f32x4*>(Qs + t * QS + d) = q_in[i] * a.q_scale;
-        *reinterpret_cast<f32x4*>(Ks + t * QS + d) = k_in[i];
+        *reinterpret_cast<f32x4*>(Qs + t * QS + d) = in.q[i] * a.q_scale;
+        *reinterpret_cast<f32x4*>(Ks + t * QS + d) = in.k[i];
       }
     }
-    *reinterpret_cast<f32x4*>(Vs + (threadIdx.x >> 4) * 68 + (threadIdx.x & 15) * 4) = v_in;
+    *reinterpret_cast<f32x4*>(Vs + (threadIdx.x >> 4) * 68 + (threadIdx.x & 15) * 4) = in.v;
     if (threadIdx.x < ML_L) {
       const int t = threadIdx.x;
       float i_log = 0.f, f_log = 0.f;
       if (t < valid) {
-        i_log = a.gates_ready ? gate_i : a.cap * tanhf((gate_i + a.i_bias[head]) / a.cap);
-        f_log = a.gates_ready ? gate_f : ml_logsigmoid(a.cap * tanhf((gate_f + a.f_bias[head]) / a.cap));
+        i_log = a.gates_ready ? in.gate_i : a.cap * tanhf((in.gate_i + a.i_bias[head]) / a.cap);
+        f_log = a.gates_ready ? in.gate_f : ml_logsigmoid(a.cap * tanhf((in.gate_f + a.f_bias[head]) / a.cap));
       }
       float F = f_log;                            // inclusive running sum over the 16 lanes
-#pragma unroll
-      for (int o = 1; o < ML_L; o <<= 1) {
-        const float up = __shfl_up(F, o, TW_WAVE);
-        if (t >= o) F += up;
-      }
+      F += ml_row_below<1>(F, 0.f);
+      F += ml_row_below<2>(F, 0.f);
+      F += ml_row_below<4>(F, 0.f);
+      F += ml_row_below<8>(F, 0.f);
       const float u = t < valid ? i_log - F : -INFINITY;
       float best = fmaxf(u, m0);                  // running maximum, m0 included
-#pragma unroll
-      for (int o = 1; o < ML_L; o <<= 1) {
-        const float up = __shfl_up(best, o, TW_WAVE);
-        if (t >= o) best = fmaxf(best, up);
-      }
+      best = fmaxf(best, ml_row_below<1>(best, -INFINITY));
+      best = fmaxf(best, ml_row_below<2>(best, -INFINITY));
+      best = fmaxf(best, ml_row_below<4>(best, -INFINITY));
+      best = fmaxf(best, ml_row_below<8>(best, -INFINITY));
       u_s[t] = u;
       g_s[t] = best;
       F_s[t] = F;
@@ -236,7 +252,7 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
       f_s[t] = expf(-(F + best));
     }
     __syncthreads();
-    if (c0 + ML_L < r1) request(c0 + ML_L);       // the next chunk's rows travel while this one is worked on
+    if (c0 + 2 * ML_L < r1) request(c0 + 2 * ML_L, in);   // (its registers are free again: two chunks' rows travel at a time)
     // ---- 2: K Q^T over this wave's share of the key elements; n0 . q_t ------------------------------------
     {
       f32x4 p = {0.f, 0.f, 0.f, 0.f};
@@ -249,8 +265,7 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
       const int t = threadIdx.x >> 4, piece = threadIdx.x & 15;
       float sum = 0.f;
       for (int d = piece; d < Dp; d += 16) sum = __fmaf_rn(n_s[d], Qs[t * QS + d], sum);
-#pragma unroll
-      for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, TW_WAVE);
+      sum = ml_row_sum(sum);
       if (piece == 0) nq_s[t] = sum;
     }
     __syncthreads();
@@ -321,6 +336,10 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(MlstmArgs a) {
     m0 = F_s[last] + g_last;
     // (no barrier here: the next iteration writes the other copy of the rows, and what it shares with this one, part, n_s
     // and nq_s, is written behind its first barrier, which every wave reaches only when it is done here)
+  };
+  for (int c0 = r0; c0 < r1; c0 += 2 * ML_L) {
+    link(c0, 0, even);
+    if (c0 + ML_L < r1) link(c0 + ML_L, 1, odd);
   }
   __syncthreads();
   if (wave_on) {
