@@ -172,14 +172,14 @@ def rufusun_config(size, layers, context):
 # the first with a dense feed-forward and the others with routed experts (16 experts of a quarter of the dense inner size,
 # two a token, beside a shared expert of that size, as in the Rufusun run, which is measured beside it). Latent attention:
 # the size's heads, 64 unrotated + 64 rotated query/key elements a head, values of the head size, a latent of 192. mLSTM:
-# the size's heads, keys and values of the head size. Windowed attention: the size's heads, key heads and window, four kept
+# the size's heads, keys and values of the head size. Windowed attention: the size's heads, key heads and window, eight kept
 # first tokens, convolutions of four taps, rotation over half of a head.
 def tadalorn_config(size, layers, context):
     width, heads, kv_heads, dim, ff, window = DESIGN_SIZES[size]
     dense = {"kind": "dense", "ff": ff}
     routed = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4}}
     latent = {"heads": heads, "dim": dim - 64, "rot_dim": 64, "vdim": dim, "kv_rank": 192, "scale": dim ** -0.5,
-              "rot": {"base": 50000.0, "dims": 64}}
+              "rot": {"base": 10000.0, "dims": 64}}
     out = []
     for i in range(layers):
         mlp = routed if i % 4 else dense
@@ -190,8 +190,8 @@ def tadalorn_config(size, layers, context):
         else:
             out.append({"type": "attention", "mlp": mlp,
                         "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "conv": 4,
-                                  "mask": {"size": window, "keep_first": 4}, "rot": {"base": 1e6, "dims": dim // 2}}})
-    return {"architecture": "Tadalorn", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+                                  "mask": {"size": window, "keep_first": 8}, "rot": {"base": 1e6, "dims": dim // 2}}})
+    return {"architecture": "Tadalorn", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
             "logit_softcap": 30.0, "layers": out}
 
 

@@ -17,6 +17,7 @@ import torch
 
 from ..cache.spec import CacheNeed, PagedKV
 from ..kernels import ops
+from ..weights.spec import ONE_PLUS_NORMAL, VECTOR, TensorSpec
 from .base import Mixer
 from .delta import StackedTaps
 from .linear import Linear
@@ -99,7 +100,6 @@ class ConvolvedWindowAttention(Mixer):
         return [self.proj, self.conv, self.o, self.position]
 
     def tensor_specs(self):
-        from ..weights.spec import ONE_PLUS_NORMAL, VECTOR, TensorSpec
         H, G, D = self.q_heads, self.kv_heads, self.dim
         return (self.proj.tensor_specs() + self.conv.tensor_specs() + self.o.tensor_specs() +
                 [TensorSpec(self.norm_names[0], (H * D,), VECTOR, ONE_PLUS_NORMAL),
