@@ -205,7 +205,8 @@ def main(argv=None):
                           **formula,
                           "cache_groups": [{"layers": len(g.slots), "kv_heads": g.spec.kv_heads,
                                             "head_dim": g.spec.head_dim, "window": g.spec.window,
-                                            **({"value_dim": g.spec.value_dim} if g.spec.value_dim else {})}
+                                            **({"value_dim": g.spec.value_dim} if g.spec.value_dim else {}),
+                                            **({"keep_first": g.spec.keep_first} if g.spec.keep_first else {})}
                                            for g in layout.groups],
                           # what a request holds besides pages: recurrent state, the last inputs of convolutions
                           "state_bytes_per_request": sum(
