@@ -313,16 +313,21 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const T* __restrict__ 
 
 // ---- combine: x[token] += its experts' rows, in the order of its choices ------------------------------------------
 // A workgroup takes 1,024 columns of a row, four a thread where rows and addresses allow 16-byte accesses.
-// weights (or null): a factor on each of the token's rows; accumulate 0: x is written, not added to.
+// weights (or null): a factor on each of the token's rows; accumulate 0: x is written, not added to. more (or null):
+// float32 [splits][n][C] partial sums of something else that belongs to the same result (a shared expert's last product
+// with its K ranges not yet added up): added here, in index order, before the experts' rows.
 template <bool VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long ld_x, const float* __restrict__ ys,
                                                           long ld_y, const int* __restrict__ pos, int C, int top,
-                                                          const float* __restrict__ weights, int accumulate) {
+                                                          const float* __restrict__ weights, int accumulate,
+                                                          const float* __restrict__ more, int splits, size_t more_stride) {
   const int row = blockIdx.x;
   const int c = blockIdx.y * 1024 + threadIdx.x * 4;
   if (c >= C) return;
   if constexpr (VEC) {
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (more)
+      for (int s = 0; s < splits; ++s) sum += *reinterpret_cast<const f32x4*>(more + s * more_stride + (size_t)row * C + c);
     for (int r = 0; r < top; ++r) {
       const f32x4 y = *reinterpret_cast<const f32x4*>(ys + (size_t)pos[(size_t)row * top + r] * ld_y + c);
       if (weights) sum += weights[(size_t)row * top + r] * y;
@@ -334,6 +339,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
   } else {
     for (int j = 0; j < 4 && c + j < C; ++j) {
       float sum = 0.f;
+      if (more)
+        for (int s = 0; s < splits; ++s) sum += more[s * more_stride + (size_t)row * C + c + j];
       for (int r = 0; r < top; ++r)
         sum += (weights ? weights[(size_t)row * top + r] : 1.f) * ys[(size_t)pos[(size_t)row * top + r] * ld_y + c + j];
       if (accumulate) x[(size_t)row * ld_x + c + j] += sum;
@@ -348,9 +355,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
 extern "C" int tw_moe_experts(int dtype, const void* h, long ld_h, const int* ids, const float* weights, int n, int top, int X,
                               const void* gate, const void* up, const void* down, int C, int Cd, int Fd, float limit,
                               int* pos, int* src_item, int* tile_expert, void* xs, void* act, float* ys, int capacity,
-                              float* x, long ld_x, int kind, int accumulate, hipStream_t stream) {
+                              float* x, long ld_x, int kind, int accumulate, const float* more, int more_splits,
+                              hipStream_t stream) {
   TW_REQUIRE(h && ids && weights && up && down && pos && src_item && tile_expert && xs && act && ys && x);
   TW_REQUIRE((kind == 0 && gate) || kind == 1);
+  TW_REQUIRE(more == nullptr || more_splits > 0);
   if (kind == 1) gate = up;            // (never read: the alignment test below wants a pointer)
   TW_REQUIRE(n >= 0 && top > 0 && C > 0 && Cd >= C && Cd % 32 == 0 && Fd > 0 && Fd % 32 == 0 && ld_h >= C && ld_x >= C);
   TW_REQUIRE((uintptr_t)xs % 16 == 0 && (uintptr_t)act % 16 == 0 && (uintptr_t)gate % 16 == 0 && (uintptr_t)up % 16 == 0 &&
@@ -434,9 +443,12 @@ extern "C" int tw_moe_experts(int dtype, const void* h, long ld_h, const int* id
     return TW_ERR_BAD_ARGUMENT;
   }
   const dim3 combine_grid(n, tw_div_up(C, 1024));
-  if (C % 4 == 0 && ld_x % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)ys % 16 == 0)
-    moe_combine_kernel<true><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top, kind == 1 ? weights : nullptr, accumulate);
+  const size_t more_stride = (size_t)n * C;
+  if (C % 4 == 0 && ld_x % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)ys % 16 == 0 && (uintptr_t)more % 16 == 0)
+    moe_combine_kernel<true><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top, kind == 1 ? weights : nullptr, accumulate,
+                                                               more, more_splits, more_stride);
   else
-    moe_combine_kernel<false><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top, kind == 1 ? weights : nullptr, accumulate);
+    moe_combine_kernel<false><<<combine_grid, 256, 0, stream>>>(x, ld_x, ys, C, pos, C, top, kind == 1 ? weights : nullptr, accumulate,
+                                                                more, more_splits, more_stride);
   return TW_LAUNCH_RESULT();
 }

@@ -71,7 +71,7 @@ _SIGNATURES = {
     "tw_head_norm_gate": (I, [I, P, L, P, L, P, P, L, I, I, I, F, I, I, P]),
     "tw_moe_route": (I, [I, P, L, P, P, I, I, I, I, I, P, P, P]),
     "tw_moe_capacity": (L, [L, I]),
-    "tw_moe_experts": (I, [I, P, L, P, P, I, I, I, P, P, P, I, I, I, F, P, P, P, P, P, P, I, P, L, I, I, P]),
+    "tw_moe_experts": (I, [I, P, L, P, P, I, I, I, P, P, P, I, I, I, F, P, P, P, P, P, P, I, P, L, I, I, P, I, P]),
     "tw_add_normed": (I, [I, P, P, L, P, I, L, P, P, I, I, F, F, P]),
     "tw_activation": (I, [I, P, L, I, I, P, I, I, P]),
     "tw_sigmoid_gate": (I, [I, P, L, P, L, I, I, I, P]),

@@ -1158,9 +1158,10 @@ def moe_blocked(w):
 MOE_KINDS = {"swish_limited": 0, "gelu": 1}
 
 
-def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch, kind="swish_limited", accumulate=True):
+def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch, kind="swish_limited", accumulate=True, more=None):
     """kind "gelu" (gate None): x[n] (+)= sum over a row's chosen experts e of weights_e * down_e(gelu(up_e h[n])), the exact
-    gelu; accumulate=False writes x instead of adding to it. kind "swish_limited": x[n] += sum over a row's chosen experts e of down_e(glu(gate_e y, up_e y)), y = round(weights * h[n]), glu the
+    gelu; accumulate=False writes x instead of adding to it; more: float32 [splits, n, C] partial sums of something that
+    belongs to the same result (a shared expert's last product), added up here as well. kind "swish_limited": x[n] += sum over a row's chosen experts e of down_e(glu(gate_e y, up_e y)), y = round(weights * h[n]), glu the
     limited swish with LIMIT. gate, up [X, Fd, Cd], down [X, C16, Fd] in h's type, zero padded (Fd, Cd: `moe_pad` of the
     sizes, C16: C rounded up to 16) and laid out by `moe_blocked`. scratch(tag, shape, dtype) hands out the step's scratch tensors."""
     n, C, ld_h = _rows(h, "h")
@@ -1176,6 +1177,9 @@ def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch, kind="swish_
           "ids and weights are [n, top]")
     nx, cx, ld_x = _rows(x, "x")
     _need(nx == n and cx == C and x.dtype == torch.float32, "x must be float32 [n, C]")
+    if more is not None:
+        _need(more.dim() == 3 and more.is_contiguous() and tuple(more.shape[1:]) == (n, C) and more.dtype == torch.float32,
+              "more must be float32 [splits, n, C]")
     capacity = moe_capacity(n * top, X)
     pos = scratch("moe.pos", (n * top,), torch.int32)
     src_item = scratch("moe.src", (capacity,), torch.int32)
@@ -1187,7 +1191,9 @@ def moe_experts(h, ids, weights, gate, up, down, limit, x, scratch, kind="swish_
                                    _dev(weights, torch.float32, "weights"), n, top, X, _dev(gate) if gate is not None else None,
                                    _dev(up), _dev(down), C, Cd, Fd,
                                    float(limit), _dev(pos), _dev(src_item), _dev(tile_expert), _dev(xs), _dev(act), _dev(ys),
-                                   capacity, _dev(x), ld_x, MOE_KINDS[kind], 1 if accumulate else 0, _stream()), "moe_experts")
+                                   capacity, _dev(x), ld_x, MOE_KINDS[kind], 1 if accumulate else 0,
+                                   _dev(more) if more is not None else None, more.shape[0] if more is not None else 0,
+                                   _stream()), "moe_experts")
     return x
 
 

@@ -199,9 +199,9 @@ def _feed_forward(prefix, C, mlp):
         return GatedFeedForward([prefix + "gate", prefix + "up", prefix + "down"], C, mlp["ff"], activation="silu", suffix="")
     shared = mlp.get("shared")
     if shared is not None:
-        # (the routed experts add to what the shared one wrote, so it finishes its sums itself)
+        # (where its last product splits K, the sums are added up by the kernel that adds up a token's experts)
         shared = PlainFeedForward([prefix + "shared.up", prefix + "shared.down"], C, shared["ff"], suffix="",
-                                  activation="gelu", defer=False)
+                                  activation="gelu")
     return RoutedExperts(prefix, C, mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"], shared=shared,
                          kind="gelu", weighting="softmax_chosen", router_bias="router.b")
 

@@ -93,9 +93,10 @@ class RoutedExperts(FeedForward):
 
     def forward(self, ctx, h, x, accumulate=True):
         n = h.shape[0]
-        if self.shared is not None:          # (with accumulate=False the shared expert writes x and the routed ones add to it)
-            if self.shared.forward(ctx, h, x, accumulate=accumulate) is not None:
-                raise RuntimeError("a shared expert must finish its sums itself")
+        # (with accumulate=False the shared expert writes x and the routed ones add to it, or it leaves the split-K sums of
+        # its last product pending and the kernel that adds up a token's experts adds those too)
+        pending = self.shared.forward(ctx, h, x, accumulate=accumulate) if self.shared is not None else None
+        wrote = self.shared is not None and pending is None
         ids = ctx.scratch("moe.ids", (n, self.top), torch.int32)
         weights = ctx.scratch("moe.weights", (n, self.top), torch.float32)
         ops.moe_route(h, self.router, self.top, ids, weights, bias=self.router_bias, weighting=self.weighting)
@@ -106,5 +107,5 @@ class RoutedExperts(FeedForward):
             rows = {"moe.pos": ctx.max_tokens * self.top, "moe.tiles": most // 16}.get(tag, most)
             return ctx.workspace.get(f"{tag}.{self.top}.{self.experts}", shape, dtype, capacity=rows)
         ops.moe_experts(h, ids, weights, self.gate, self.up, self.down, self.limit, x, scratch, kind=self.kind,
-                        accumulate=accumulate or self.shared is not None)
+                        accumulate=accumulate or wrote, more=pending)
         return None
