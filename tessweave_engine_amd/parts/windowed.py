@@ -10,6 +10,11 @@
 Query head a reads key head a // (heads / kv_heads). Keys and values are paged like every attention layer's (a windowed
 cache group that never gives back the pages of the kept first tokens); the convolutions' last inputs are a float32
 state of the cache slot. Convolutions, norms, angles, scores and the softmax are float32 in both precisions.
+
+Two attention kernels serve it. The one that knows kept first keys (`ops.attn_mixed`) takes one-token sequences always, and
+prompt portions whenever some query's window has passed a kept token. Portions of steps in which that cannot matter (no
+kept tokens, or every sequence of the step still shorter than the window, so that every earlier key is seen anyway)
+run the engine's prompt kernel (`ops.attn_prefill`, with the sink), which is several times as fast; both read the same pages.
 """
 from __future__ import annotations
 
@@ -28,9 +33,10 @@ def _round_up(v, m):
 
 
 def mixed_attention(ctx, q, keys, values, group, out, q_heads, kv_heads, value_dev, scale, window=0, keep_first=0, sink=None,
-                    tag="attn.window"):
-    """The step's one-token sequences and its prompt portions through the attention kernel that takes a window, kept
-    first keys and a sink. keys [pages, kv_heads, page, key_dev], values [pages, kv_heads, value_dev, page]."""
+                    tag="attn.window", portions=True):
+    """The step's one-token sequences and (unless portions=False) its prompt portions through the attention kernel that
+    takes a window, kept first keys and a sink. keys [pages, kv_heads, page, key_dev], values [pages, kv_heads,
+    value_dev, page]."""
     common = dict(window=window, keep_first=keep_first, sink=sink)
     span = window + _round_up(keep_first, 16) if window else 0        # most keys a query walks
     if ctx.n_decode:
@@ -48,7 +54,7 @@ def mixed_attention(ctx, q, keys, values, group, out, q_heads, kv_heads, value_d
             ws = ctx.workspace.get(tag + ".split", (floats,), torch.float32)
         ops.attn_mixed(q, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode, 1, out, q_heads,
                        kv_heads, scale, splits=splits, workspace=ws, **common)
-    if ctx.n_seqs > ctx.n_decode:
+    if portions and ctx.n_seqs > ctx.n_decode:
         n_seqs = ctx.n_seqs - ctx.n_decode
         longest = min(ctx.max_kv_len, span + ctx.max_q_len) if window else ctx.max_kv_len
         splits = ops.attn_mixed_prefill_splits(ctx.n_tokens - ctx.n_decode, n_seqs, longest)
@@ -131,14 +137,27 @@ class ConvolvedWindowAttention(Mixer):
         self.conv.forward(ctx, run, proj[:, :channels], out32=qk)
         cos, sin = self.position.tables(ctx)
         keys, values, g = ctx.cache.keys_values(run.cache_slot)
+        pages = values
         values = values.view(values.shape[0], G, Dp, ctx.cache.page_size)
         group = ctx.groups[g]
         q = ctx.scratch("window.q", (n, H * Dp))
         ops.qk_finish(qk, 0, H * D, self.q_weight, self.k_weight, cos, sin, q, keys, values, group.slot_mapping, H, G, D,
                       self.position.rotary_dim, self.eps, adjacent=self.position.pairing == "adjacent")
         out = ctx.scratch("window.out", (n, H * Dp))
-        mixed_attention(ctx, q, keys, values, group, out, H, G, Dp, self.scale, window=self.window or 0,
-                        keep_first=self.keep_first, sink=self.sink)
+        window, portions = self.window or 0, ctx.n_seqs - ctx.n_decode
+        all_seen = not window or ctx.max_kv_len <= window          # no query of the step has a key behind its window
+        fast = portions > 0 and (all_seen or self.keep_first == 0)
+        mixed_attention(ctx, q, keys, values, group, out, H, G, Dp, self.scale, window=window, keep_first=self.keep_first,
+                        sink=self.sink, portions=not fast)
+        if fast:
+            seen = 0 if all_seen else window
+            longest = min(ctx.max_kv_len, seen + ctx.max_q_len) if seen else ctx.max_kv_len
+            split = ops.attn_prefill_split(portions, H, G, ctx.max_q_len, longest)
+            ws = None
+            if split[0] > 1:
+                ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, Dp, split[0]),), torch.float32)
+            ops.attn_prefill(q, keys, pages, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode, portions, ctx.max_q_len,
+                             out, H, G, Dp, self.scale, window=seen, split=split, workspace=ws, sink=self.sink)
         ops.sigmoid_gate(out, proj[:, self.gate_col:])
         if ctx.defer_sums and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # whoever norms next adds them up
