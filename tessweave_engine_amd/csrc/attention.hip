@@ -72,6 +72,9 @@ struct AttnArgs {
                              // chunks a tile can have; max_chunks == 1: a tile's keys are never split
   const float* sink;         // prefill only. [q_heads] or null: exp(sink_h) more in head h's denominator (a score of its
                              // own, not scaled, with no key and no value)
+  float* stats;              // prefill only. [token rows][q_heads][2] or null: what a row's softmax was taken against (the
+                             // reference, as a scaled score in natural units) and its sum relative to that, for whoever adds
+                             // more keys to the row afterwards
 };
 
 // Per-wave online-softmax state for one 16-row tile. Lane (r, g) belongs to row r.
@@ -625,6 +628,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 
   if (!row_ok) return;
   const float inv = tile.l > 0.f ? 1.f / tile.l : 0.f;
+  if (a.stats && g == 0) {
+    float* st = a.stats + ((size_t)(token0 + tok) * a.q_heads + head) * 2;
+    st[0] = tile.m == -INFINITY ? 0.f : tile.m;
+    st[1] = tile.l;
+  }
   T* dst = (T*)a.out + (size_t)(token0 + tok) * a.ldo + (size_t)head * D;
 #pragma unroll
   for (int dt = 0; dt < DTMAX; ++dt)
@@ -1342,6 +1350,11 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   for (int rt = 0; rt < RT; ++rt) {
     if (!row_ok[rt]) continue;
     const float inv = l[rt] > 0.f ? 1.f / l[rt] : 0.f;
+    if (a.stats && g == 0) {
+      float* st = a.stats + ((size_t)(token0 + tok[rt]) * a.q_heads + head[rt]) * 2;
+      st[0] = m_use[rt] * 0.69314718055994530942f;           // (kept in the log2 domain here)
+      st[1] = l[rt];
+    }
     bf16_t* dst = (bf16_t*)a.out + (size_t)(token0 + tok[rt]) * a.ldo + (size_t)head[rt] * D;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
@@ -1392,6 +1405,11 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnArgs a) {
       for (int e = 0; e < 4; ++e) o[e] += x[e] * w;
     }
     if (a.sink) l_all += __builtin_amdgcn_exp2f(fmaf(a.sink[head], 1.44269504088896340736f, -m_use));
+    if (a.stats && grp == 0) {
+      float* st = a.stats + ((size_t)(token0 + tok) * a.q_heads + head) * 2;
+      st[0] = m_use * 0.69314718055994530942f;
+      st[1] = l_all;
+    }
     const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
     bf16_t packed[4];
 #pragma unroll
@@ -1576,7 +1594,7 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
   a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = splits;
-  a.sink = nullptr;
+  a.sink = nullptr; a.stats = nullptr;
   TW_REQUIRE(softcap >= 0.f);
   a.softcap = softcap;
   a.part_o = nullptr; a.part_ml = nullptr;
@@ -1626,9 +1644,10 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
                                const int* kv_len, int seq0, int n_seqs, int max_q_len, void* out,
                                long ldo, float* workspace, long workspace_floats, int n_tokens, int max_chunks,
                                int kv_chunk, int tile_rows, int q_heads, int kv_heads, int head_dim, int page_size,
-                               int window, float scale, float softcap, int generic, const float* sink, hipStream_t stream) {
+                               int window, float scale, float softcap, int generic, const float* sink, float* stats,
+                               hipStream_t stream) {
   AttnArgs a;
-  a.sink = sink;
+  a.sink = sink; a.stats = stats;
   TW_REQUIRE(tile_rows == 0 || tile_rows == 64 || tile_rows == 128);
   a.tile_rows = tile_rows;
   a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
@@ -1659,4 +1678,105 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
   if (dtype == TW_DTYPE_F32) return prefill_launch<float>(a, n_seqs, max_q_len, generic, stream);
   if (dtype == TW_DTYPE_BF16) return prefill_launch<bf16_t>(a, n_seqs, max_q_len, generic, stream);
   return TW_ERR_BAD_ARGUMENT;
+}
+
+// =====================================================================================
+// Keys in front of a window. A prompt kernel above has run with a window and has left, per (token, head), the normalised
+// output and the row's statistics (reference, sum). This kernel adds what the window left out and the design still sees:
+// the sequence's first `keep` keys as far as they lie BEFORE the row's window (positions j < min(keep, t - window + 1)),
+// and a sink (exp(sink_h) more in the denominator), and writes the row's output anew:
+//   out = (out_w l_w e^(m_w - m) + sum_kept e^(s_j - m) v_j) / (l_w e^(m_w - m) + sum_kept e^(s_j - m) + e^(sink - m)).
+// One wave a (token, head); a lane holds head_dim / 64 elements; scores and sums are float32. The kept keys are few
+// (a handful of tokens), so this is a small fraction of the window's work.
+// =====================================================================================
+struct KeptArgs {
+  const void* q; long ldq;
+  const void* keys; const void* values;
+  const int* block_table; int table_stride;
+  const int* q_start; const int* kv_len;
+  int seq0, n_seqs;
+  void* out; long ldo;
+  const float* stats;      // [token rows][q_heads][2]
+  const float* sink;       // [q_heads] or null
+  int q_heads, kv_heads, head_dim, page_size, window, keep;
+  float scale;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_kept_keys_kernel(KeptArgs a, int row0, int n_rows) {
+  const int lane = threadIdx.x & 63;
+  const long unit = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (unit >= (long)n_rows * a.q_heads) return;
+  const int row = row0 + (int)(unit / a.q_heads), head = (int)(unit % a.q_heads);
+  // the row's sequence: the launch's sequences own consecutive rows (a handful of sequences: a walk over them)
+  int seq = a.seq0;
+  while (seq + 1 < a.seq0 + a.n_seqs && row >= a.q_start[seq + 1]) ++seq;
+  const int q0 = a.q_start[seq], q_len = a.q_start[seq + 1] - q0;
+  const int t = a.kv_len[seq] - q_len + (row - q0);
+  const int n_kept = a.window > 0 ? min(a.keep, t - a.window + 1) : 0;       // kept keys before the row's window
+  const int D = a.head_dim, P = a.page_size, kvh = head / (a.q_heads / a.kv_heads);
+  constexpr int PER = 4;                                    // head_dim <= 256
+  float qv[PER], o[PER];
+  const T* q = (const T*)a.q + (size_t)row * a.ldq + (size_t)head * D;
+  T* out = (T*)a.out + (size_t)row * a.ldo + (size_t)head * D;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int d = lane + 64 * i;
+    qv[i] = d < D ? tw_to_float(q[d]) : 0.f;
+    o[i] = 0.f;
+  }
+  const float* st = a.stats + ((size_t)row * a.q_heads + head) * 2;
+  const float m_w = st[1] > 0.f ? st[0] : -INFINITY, l_w = st[1];
+  float m = a.sink ? fmaxf(m_w, a.sink[head]) : m_w, l = 0.f;
+  if (m == -INFINITY) m = 0.f;
+  const int* table = a.block_table + (size_t)seq * a.table_stride;
+  for (int j = 0; j < n_kept; ++j) {
+    const int page = table[j / P], at = j % P;
+    const T* k = (const T*)a.keys + (((size_t)page * a.kv_heads + kvh) * P + at) * D;
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int d = lane + 64 * i;
+      if (d < D) s = __fmaf_rn(qv[i], tw_to_float(k[d]), s);
+    }
+    s = tw_wave_sum(s) * a.scale;
+    const float m_new = fmaxf(m, s);
+    const float alpha = expf(m - m_new), p = expf(s - m_new);
+    const T* v = (const T*)a.values + ((size_t)page * a.kv_heads + kvh) * D * P + at;
+    l = l * alpha + p;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int d = lane + 64 * i;
+      if (d < D) o[i] = __fmaf_rn(p, tw_to_float(v[(size_t)d * P]), o[i] * alpha);
+    }
+    m = m_new;
+  }
+  const float w = m_w == -INFINITY ? 0.f : l_w * expf(m_w - m);      // what the window's sum weighs against the new reference
+  const float total = w + l + (a.sink ? expf(a.sink[head] - m) : 0.f);
+  const float inv = total > 0.f ? 1.f / total : 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) out[d] = tw_from_float<T>((tw_to_float(out[d]) * w + o[i]) * inv);
+  }
+}
+
+// Rows row0 .. row0 + n_rows - 1 belong to sequences seq0 .. seq0 + n_seqs - 1, in order.
+extern "C" int tw_attn_kept_keys(int dtype, const void* q, long ldq, const void* keys, const void* values,
+                                 const int* block_table, int table_stride, const int* q_start, const int* kv_len, int seq0,
+                                 int n_seqs, int row0, int n_rows, void* out, long ldo, const float* stats, const float* sink,
+                                 int q_heads, int kv_heads, int head_dim, int page_size, int window, int keep, float scale,
+                                 hipStream_t stream) {
+  TW_REQUIRE(q && keys && values && block_table && q_start && kv_len && out && stats);
+  TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && row0 >= 0 && n_rows >= 0 && window >= 0 && keep >= 0);
+  TW_REQUIRE(q_heads >= 1 && kv_heads >= 1 && q_heads % kv_heads == 0 && head_dim >= 1 && head_dim <= 256 && page_size > 0);
+  TW_REQUIRE(ldq >= (long)q_heads * head_dim && ldo >= (long)q_heads * head_dim && table_stride > 0);
+  if (n_seqs == 0 || n_rows == 0) return 0;
+  KeptArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, seq0, n_seqs, out, ldo, stats, sink,
+             q_heads, kv_heads, head_dim, page_size, window, keep, scale};
+  const int blocks = tw_div_up((long)n_rows * q_heads, 4);
+  if (dtype == TW_DTYPE_BF16) attn_kept_keys_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, row0, n_rows);
+  else if (dtype == TW_DTYPE_F32) attn_kept_keys_kernel<float><<<blocks, 256, 0, stream>>>(a, row0, n_rows);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
 }

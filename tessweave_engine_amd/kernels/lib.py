@@ -36,7 +36,8 @@ _SIGNATURES = {
     "tw_attn_decode": (I, [I, P, L, P, P, P, I, P, P, I, I, P, L, P, L, I, I, I, I, I, F, F, I, I, P]),
     "tw_attn_prefill_split": (I, [I, I, I, I, I, I, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "tw_attn_prefill_workspace_floats": (L, [I, I, I, I]),
-    "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P, P]),
+    "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P, P, P]),
+    "tw_attn_kept_keys": (I, [I, P, L, P, P, P, I, P, P, I, I, I, I, P, L, P, P, I, I, I, I, I, I, F, P]),
     "tw_add_table_rows": (I, [I, P, P, P, I, I, I, P, P]),
     "tw_causal_conv": (I, [I, I, P, L, P, F, P, P, F, P, P, P, P, P, P, L, P, L, I, I, I, I, P, I, P]),
     "tw_gated_recurrence_workspace_floats": (L, [I, I, I]),

@@ -433,11 +433,13 @@ def attn_prefill_workspace_floats(n_tokens, q_heads, head_dim, max_chunks):
 
 
 def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_q_len, out, q_heads,
-                 kv_heads, head_dim, scale, window=0, generic=False, split=None, workspace=None, softcap=0.0, sink=None):
+                 kv_heads, head_dim, scale, window=0, generic=False, split=None, workspace=None, softcap=0.0, sink=None,
+                 stats=None):
     """Attention of sequences seq0..seq0+n_seqs-1 with up to max_q_len query tokens each.
 
     sink float32 [q_heads]: exp(sink_h) more in head h's softmax denominator (a score of its own, not scaled, with
-    no key and no value).
+    no key and no value). stats float32 [rows of q, q_heads, 2]: gets what each row's softmax was taken against (a scaled
+    score) and the row's sum relative to it, for `attn_kept_keys`.
 
     split = (max_chunks, kv_chunk[, tile_rows]) from attn_prefill_split with a float32 workspace of
     attn_prefill_workspace_floats(rows of q, ...) lets the fast bfloat16 kernel cut long key ranges
@@ -446,6 +448,8 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
     _need(sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == q_heads), "sink must be float32 [q_heads]")
+    _need(stats is None or (stats.dtype == torch.float32 and stats.is_contiguous() and stats.numel() >= q.shape[0] * q_heads * 2),
+          "stats must be float32 [rows, q_heads, 2]")
     max_chunks, kv_chunk, ws_ptr, ws_floats = 1, 0, None, 0
     tile_rows = int(split[2]) if split is not None and len(split) > 2 else 0
     if split is not None and split[0] > 1:
@@ -458,7 +462,28 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
                                     seq0, n_seqs, int(max_q_len), _dev(out), ldo, ws_ptr, ws_floats, q.shape[0],
                                     max_chunks, kv_chunk, tile_rows, q_heads, kv_heads, head_dim,
                                     keys.shape[2], int(window or 0), float(scale), float(softcap or 0.0),
-                                    1 if generic else 0, _dev(sink) if sink is not None else None, _stream()), "attn_prefill")
+                                    1 if generic else 0, _dev(sink) if sink is not None else None,
+                                    _dev(stats) if stats is not None else None, _stream()), "attn_prefill")
+    return out
+
+
+def attn_kept_keys(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, row0, n_rows, out, stats, q_heads, kv_heads,
+                   head_dim, scale, window, keep_first, sink=None):
+    """Completes rows row0 .. row0 + n_rows - 1 (those of sequences seq0 .. seq0 + n_seqs - 1, in order) of a windowed
+    `attn_prefill` that left `stats`: adds the sequence's first keep_first keys as far as they lie before a row's window,
+    and the sink, and writes out anew. Same cache layout as `attn_prefill`."""
+    ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
+    _need(stats.dtype == torch.float32 and stats.is_contiguous() and stats.numel() >= q.shape[0] * q_heads * 2,
+          "stats must be float32 [rows, q_heads, 2]")
+    _need(row0 + n_rows <= q.shape[0] and seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0],
+          "rows or sequences exceed the step")
+    _need(sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == q_heads), "sink must be float32 [q_heads]")
+    check(library().tw_attn_kept_keys(dtype_id(q.dtype), _dev(q), ldq, _dev(keys), _dev(values),
+                                      _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
+                                      _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"), int(seq0),
+                                      int(n_seqs), int(row0), int(n_rows), _dev(out), ldo, _dev(stats),
+                                      _dev(sink) if sink is not None else None, q_heads, kv_heads, head_dim, keys.shape[2],
+                                      int(window or 0), int(keep_first or 0), float(scale), _stream()), "attn_kept_keys")
     return out
 
 

@@ -11,10 +11,10 @@ Query head a reads key head a // (heads / kv_heads). Keys and values are paged l
 cache group that never gives back the pages of the kept first tokens); the convolutions' last inputs are a float32
 state of the cache slot. Convolutions, norms, angles, scores and the softmax are float32 in both precisions.
 
-Two attention kernels serve it. The one that knows kept first keys (`ops.attn_mixed`) takes one-token sequences always, and
-prompt portions whenever some query's window has passed a kept token. Portions of steps in which that cannot matter (no
-kept tokens, or every sequence of the step still shorter than the window, so that every earlier key is seen anyway)
-run the engine's prompt kernel (`ops.attn_prefill`, with the sink), which is several times as fast; both read the same pages.
+Two attention kernels serve it, both on the same pages. One-token sequences run the kernel that knows kept first keys
+(`ops.attn_mixed`). Prompt portions run the engine's prompt kernel (`ops.attn_prefill`) over the window, with the sink;
+in steps in which some query's window may have passed a kept token the prompt kernel leaves each row's softmax statistics
+instead, and a small kernel (`ops.attn_kept_keys`) adds the kept keys in front of the row's window, and the sink.
 """
 from __future__ import annotations
 
@@ -145,19 +145,25 @@ class ConvolvedWindowAttention(Mixer):
                       self.position.rotary_dim, self.eps, adjacent=self.position.pairing == "adjacent")
         out = ctx.scratch("window.out", (n, H * Dp))
         window, portions = self.window or 0, ctx.n_seqs - ctx.n_decode
-        all_seen = not window or ctx.max_kv_len <= window          # no query of the step has a key behind its window
-        fast = portions > 0 and (all_seen or self.keep_first == 0)
         mixed_attention(ctx, q, keys, values, group, out, H, G, Dp, self.scale, window=window, keep_first=self.keep_first,
-                        sink=self.sink, portions=not fast)
-        if fast:
+                        sink=self.sink, portions=False)
+        if portions:
+            all_seen = not window or ctx.max_kv_len <= window      # no query of the step has a key behind its window
             seen = 0 if all_seen else window
+            kept = bool(seen and self.keep_first)                  # some window may have passed a kept token
             longest = min(ctx.max_kv_len, seen + ctx.max_q_len) if seen else ctx.max_kv_len
             split = ops.attn_prefill_split(portions, H, G, ctx.max_q_len, longest)
             ws = None
             if split[0] > 1:
                 ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, Dp, split[0]),), torch.float32)
+            stats = ctx.scratch("window.stats", (n, H, 2), torch.float32) if kept else None
             ops.attn_prefill(q, keys, pages, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode, portions, ctx.max_q_len,
-                             out, H, G, Dp, self.scale, window=seen, split=split, workspace=ws, sink=self.sink)
+                             out, H, G, Dp, self.scale, window=seen, split=split, workspace=ws,
+                             sink=None if kept else self.sink, stats=stats)
+            if kept:       # the kept keys in front of the rows' windows, and the sink
+                first_row = ctx.h_q_start[ctx.n_decode]
+                ops.attn_kept_keys(q, keys, pages, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode, portions, first_row,
+                                   n - first_row, out, stats, H, G, Dp, self.scale, window, self.keep_first, sink=self.sink)
         ops.sigmoid_gate(out, proj[:, self.gate_col:])
         if ctx.defer_sums and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # whoever norms next adds them up

@@ -34,7 +34,7 @@ from tadalorn_util import (CONFIGS, Driver, attention, config, dense, latent, ma
 pytestmark = pytest.mark.gpu
 
 BAR = {"float32": 2e-5, "bfloat16": 3e-2}
-CLOSE = 0.1
+CLOSE = 0.25         # a router margin under this may go the other way in bfloat16 (its logits carry a few per cent of their spread)
 LENGTHS = {"odd": (61, 23, 9, 150, 1), "wide": (70, 12, 33, 101, 2), "one": (40, 7, 90)}
 
 
@@ -121,16 +121,19 @@ def paged(k, v, page, order_seed, device, dtype, dim_dev):
     return keys, values, table, slots
 
 
+@pytest.mark.parametrize("portions", ["windowed_kernel", "prompt_kernel_then_kept_keys"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,G,D,rot,window,keep,page", [(4, 2, 24, 16, 9, 3, 4), (8, 8, 32, 32, 64, 0, 16), (4, 1, 64, 32, 5, 20, 8),
                                                         (2, 2, 16, 0, 33, 1, 16), (6, 3, 40, 8, 16, 16, 4), (3, 3, 128, 128, 40, 4, 16),
                                                         (16, 4, 32, 16, 24, 2, 8), (12, 12, 16, 8, 10, 17, 4), (24, 8, 16, 16, 31, 5, 16),
                                                         (32, 4, 64, 32, 48, 1, 16)])
-def test_window_with_kept_first_keys_and_a_sink_made_sharp(device, dtype, H, G, D, rot, window, keep, page):
+def test_window_with_kept_first_keys_and_a_sink_made_sharp(device, dtype, H, G, D, rot, window, keep, page, portions):
     """Whole-row norms, rotation of pairs, cache write and the attention kernel, against the plain softmax over the
     plain mask. Every query row is made to point at ONE key with a large score: the key just inside its window, the one
     just outside, the last kept key, the first one not kept, the first token, itself. A key seen wrongly or lost moves
-    its row by the size of a value. A prompt portion behind a cached history, then single tokens."""
+    its row by the size of a value. A prompt portion behind a cached history, then single tokens. The portions run the
+    windowed kernel, or the engine's prompt kernel over the window followed by the kernel that adds the kept keys in front
+    of it and the sink; single tokens always the windowed kernel."""
     from tessweave_engine_amd.kernels import ops
     T, eps, scale = 150, 1e-5, 0.5
     g = torch.Generator().manual_seed(H * D + window)
@@ -180,8 +183,17 @@ def test_window_with_kept_first_keys_and_a_sink_made_sharp(device, dtype, H, G, 
     bt = ints([table + [-1] * (width - len(table))], device)
     first = 100                                              # a portion of 100 - 37 tokens behind 37 cached ones, then single tokens
     for lo, hi in [(0, 37), (37, first)] + [(t, t + 1) for t in range(first, T)]:
-        ops.attn_mixed(q[lo:hi], keys, values, bt, ints([0, hi - lo], device), ints([hi], device), 0, 1, hi - lo, out[lo:hi], H, G,
-                       scale, window=window, keep_first=keep, sink=sink)
+        starts, lens = ints([0, hi - lo], device), ints([hi], device)
+        if hi - lo > 1 and portions != "windowed_kernel":
+            stats = torch.full((hi - lo, H, 2), float("nan"), device=device)
+            pages = values.view(values.shape[0], G, page, Dp)                 # (the same bytes: how the prompt kernels are handed them)
+            ops.attn_prefill(q[lo:hi], keys, pages, bt, starts, lens, 0, 1, hi - lo, out[lo:hi], H, G, Dp, scale, window=window,
+                             stats=stats)
+            ops.attn_kept_keys(q[lo:hi], keys, pages, bt, starts, lens, 0, 1, 0, hi - lo, out[lo:hi], stats, H, G, Dp, scale,
+                               window, keep, sink=sink)
+        else:
+            ops.attn_mixed(q[lo:hi], keys, values, bt, starts, lens, 0, 1, hi - lo, out[lo:hi], H, G,
+                           scale, window=window, keep_first=keep, sink=sink)
     got = out.view(T, H, Dp)[:, :, :D].double().cpu()
     assert torch.isfinite(out.view(T, H, Dp)[:, :, :D]).all()
     tol = 1e-4 if dtype == "float32" else 6e-2
