@@ -1702,6 +1702,20 @@ struct KeptArgs {
   float scale;
 };
 
+// Sum over a wave by DPP rotations inside the rows of 16 lanes, then the lane swaps across the four rows: no trip through
+// the LDS crossbar in the chain of a key's score.
+template <int CTRL>
+__device__ __forceinline__ float kept_row_turned(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float kept_wave_sum(float v) {
+  v += kept_row_turned<0x128>(v);
+  v += kept_row_turned<0x124>(v);
+  v += kept_row_turned<0x122>(v);
+  v += kept_row_turned<0x121>(v);
+  return tw_rows_sum(v);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void attn_kept_keys_kernel(KeptArgs a, int row0, int n_rows) {
   const int lane = threadIdx.x & 63;
@@ -1739,7 +1753,7 @@ __global__ __launch_bounds__(256) void attn_kept_keys_kernel(KeptArgs a, int row
       const int d = lane + 64 * i;
       if (d < D) s = __fmaf_rn(qv[i], tw_to_float(k[d]), s);
     }
-    s = tw_wave_sum(s) * a.scale;
+    s = kept_wave_sum(s) * a.scale;
     const float m_new = fmaxf(m, s);
     const float alpha = expf(m - m_new), p = expf(s - m_new);
     const T* v = (const T*)a.values + ((size_t)page * a.kv_heads + kvh) * D * P + at;
