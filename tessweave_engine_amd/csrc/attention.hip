@@ -1744,24 +1744,43 @@ __global__ __launch_bounds__(256) void attn_kept_keys_kernel(KeptArgs a, int row
   float m = a.sink ? fmaxf(m_w, a.sink[head]) : m_w, l = 0.f;
   if (m == -INFINITY) m = 0.f;
   const int* table = a.block_table + (size_t)seq * a.table_stride;
-  for (int j = 0; j < n_kept; ++j) {
-    const int page = table[j / P], at = j % P;
+  typedef typename KeyQuad<T>::Type Quad;
+  // four kept keys at a time (they share a page: pages hold a multiple of four keys): their scores, one step of the
+  // running softmax, then every lane's elements of their four values in one load (values lie transposed inside a page)
+  for (int j0 = 0; j0 < n_kept; j0 += 4) {
+    const int page = table[j0 / P], at = j0 % P;
     const T* k = (const T*)a.keys + (((size_t)page * a.kv_heads + kvh) * P + at) * D;
-    float s = 0.f;
+    float s[4];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int d = lane + 64 * i;
-      if (d < D) s = __fmaf_rn(qv[i], tw_to_float(k[d]), s);
+    for (int e = 0; e < 4; ++e) {
+      float dot = 0.f;
+      if (j0 + e < n_kept) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int d = lane + 64 * i;
+          if (d < D) dot = __fmaf_rn(qv[i], tw_to_float(k[(size_t)e * D + d]), dot);
+        }
+      }
+      s[e] = j0 + e < n_kept ? kept_wave_sum(dot) * a.scale : -INFINITY;
     }
-    s = kept_wave_sum(s) * a.scale;
-    const float m_new = fmaxf(m, s);
-    const float alpha = expf(m - m_new), p = expf(s - m_new);
+    const float m_new = fmaxf(fmaxf(m, fmaxf(s[0], s[1])), fmaxf(s[2], s[3]));
+    const float alpha = expf(m - m_new);
+    float p[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) p[e] = s[e] == -INFINITY ? 0.f : expf(s[e] - m_new);
+    l = l * alpha + p[0] + p[1] + p[2] + p[3];
     const T* v = (const T*)a.values + ((size_t)page * a.kv_heads + kvh) * D * P + at;
-    l = l * alpha + p;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int d = lane + 64 * i;
-      if (d < D) o[i] = __fmaf_rn(p, tw_to_float(v[(size_t)d * P]), o[i] * alpha);
+      if (d < D) {
+        const Quad vq = *reinterpret_cast<const Quad*>(v + (size_t)d * P);
+        float sum = o[i] * alpha;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (j0 + e < n_kept) sum = __fmaf_rn(p[e], tw_to_float(vq[e]), sum);
+        o[i] = sum;
+      }
     }
     m = m_new;
   }
@@ -1784,7 +1803,7 @@ extern "C" int tw_attn_kept_keys(int dtype, const void* q, long ldq, const void*
   TW_REQUIRE(q && keys && values && block_table && q_start && kv_len && out && stats);
   TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && row0 >= 0 && n_rows >= 0 && window >= 0 && keep >= 0);
   TW_REQUIRE(q_heads >= 1 && kv_heads >= 1 && q_heads % kv_heads == 0 && head_dim >= 1 && head_dim <= 256 && page_size > 0);
-  TW_REQUIRE(ldq >= (long)q_heads * head_dim && ldo >= (long)q_heads * head_dim && table_stride > 0);
+  TW_REQUIRE(ldq >= (long)q_heads * head_dim && ldo >= (long)q_heads * head_dim && table_stride > 0 && page_size % 4 == 0);
   if (n_seqs == 0 || n_rows == 0) return 0;
   KeptArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, seq0, n_seqs, out, ldo, stats, sink,
              q_heads, kv_heads, head_dim, page_size, window, keep, scale};
